@@ -79,7 +79,11 @@ class CacheGroup:
         self.v: Dict[int, object] = {}
 
     def bytes_per_token(self, element_size: int) -> int:
-        return 2 * len(self.runs) * self.need.num_kv_heads * self.need.head_dim * element_size
+        return len(self.runs) * self.need.num_kv_heads * (self.need.head_dim + self.need.value_dim) * element_size
+
+    def kept_blocks(self) -> int:
+        """Leading blocks that a window never passes: they hold positions that are read for ever."""
+        return -(-self.need.keep_first // self.page_size) if self.need.window is not None else 0
 
 
 class CacheManager:
@@ -142,10 +146,11 @@ class CacheManager:
         for g in self.groups:
             # one page more than the pool hands out: `scratch_page`, where rows that only pad a batch write
             shape = (g.pool.num_pages + 1, g.need.num_kv_heads, g.page_size, g.need.head_dim)
+            v_shape = shape[:3] + (g.need.value_dim,)
             for run in g.runs:
                 # zeroed: masked slots must hold finite values
                 g.k[run] = torch.zeros(shape, dtype=rt.cache_dtype, device=rt.device)
-                g.v[run] = torch.zeros(shape, dtype=rt.cache_dtype, device=rt.device)
+                g.v[run] = torch.zeros(v_shape, dtype=rt.cache_dtype, device=rt.device)
         for run, need in self.state_needs.items():
             dtype = {"float32": torch.float32, "bfloat16": torch.bfloat16}[need.dtype]
             # one slot more than requests: `scratch_slot`
@@ -236,7 +241,7 @@ class CacheManager:
             table = req.tables[g.index] if req is not None else []
             need = max(0, -(-budget_tokens // g.page_size) - len(table))
             if g.need.window is not None:
-                most = -(-(g.need.window - 1 + step_tokens) // g.page_size) + 1
+                most = -(-(g.need.window - 1 + step_tokens) // g.page_size) + 1 + g.kept_blocks()
                 held = sum(1 for page in table if page >= 0)
                 need = min(need, max(0, most - held))
             out.append(need)
@@ -325,7 +330,7 @@ class CacheManager:
                 continue
             first_needed = max(0, req.length - window + 1)
             table = req.tables[g.index]
-            for block in range(min(first_needed // g.page_size, len(table))):
+            for block in range(g.kept_blocks(), min(first_needed // g.page_size, len(table))):
                 if table[block] >= 0:
                     g.pool.release(table[block])
                     table[block] = -1

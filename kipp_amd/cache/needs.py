@@ -11,11 +11,20 @@ class KVNeed:
     None: every key is kept; W: only the last W positions are ever read, so
     pages wholly behind the window are given back.  `page_size` None: pages of
     the engine's size; P: this mixer's runs keep their keys in pages of P tokens
-    (runs that ask for the same form a group with a pool of its own)."""
+    (runs that ask for the same form a group with a pool of its own).
+    `v_head_dim` None: values are as wide as keys; D: values have D numbers a head.
+    `keep_first` F (with a window): positions below F are read for ever, so the
+    pages that hold them are never given back while the request lives."""
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     page_size: Optional[int] = None
+    v_head_dim: Optional[int] = None
+    keep_first: int = 0
+
+    @property
+    def value_dim(self) -> int:
+        return self.head_dim if self.v_head_dim is None else self.v_head_dim
 
 
 @dataclass(frozen=True)

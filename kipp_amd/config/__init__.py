@@ -1,7 +1,7 @@
 """Typed configurations and the architecture registry.
 
-`load_config(model_dir)` reads config.json, looks `architectures[0]` up in the
-registry and returns (family, typed config).  A family is what an architecture
+`load_config(model_dir)` reads config.json, looks `architectures[0]` (or the
+one name under `architecture`) up in the registry and returns (family, typed config).  A family is what an architecture
 registers: how to read its config.json keys and how to turn the typed config
 into a `ModelSpec` (the decoder as data).
 """
@@ -13,8 +13,8 @@ from dataclasses import dataclass
 from typing import Callable, Dict
 
 from .specs import (AttentionSpec, ConfigError, EmbeddingSpec, GatedMLPSpec,
-                    HeadSpec, LayerRun, LayerSpec, ModelSpec, NoPositionSpec,
-                    RMSNormSpec, RopeSpec)
+                    HeadSpec, LayerRun, LayerSpec, MixedHeadAttentionSpec, ModelSpec,
+                    NoPositionSpec, OnePlusRMSNormSpec, RMSNormSpec, RopeSpec)
 
 
 @dataclass(frozen=True)
@@ -52,8 +52,10 @@ def parse_config(d: dict):
     if not isinstance(d, dict):
         raise ConfigError("config.json must hold a JSON object")
     archs = d.get("architectures")
+    if archs is None and isinstance(d.get("architecture"), str):
+        archs = [d["architecture"]]         # a configuration that names its one architecture directly
     if not isinstance(archs, list) or len(archs) != 1 or not isinstance(archs[0], str):
-        raise ConfigError("config.json architectures: expected a list with one name")
+        raise ConfigError("config.json architectures: expected a list with one name (or architecture: a name)")
     family = get_architecture(archs[0])
     return family, family.parse(d)
 
@@ -91,3 +93,8 @@ from . import qwen3 as _qwen3  # noqa: E402
 
 register_architecture(_qwen3.ARCHITECTURE, _qwen3.Qwen3Config.from_dict)
 Qwen3Config = _qwen3.Qwen3Config
+
+from . import tobinex as _tobinex  # noqa: E402
+
+register_architecture(_tobinex.ARCHITECTURE, _tobinex.TobinexConfig.from_dict)
+TobinexConfig = _tobinex.TobinexConfig

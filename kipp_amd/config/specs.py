@@ -30,6 +30,17 @@ class RMSNormSpec:
 
 
 @dataclass(frozen=True)
+class OnePlusRMSNormSpec:
+    """y = x * rsqrt(mean(x^2) + eps) * (1 + w): the tensor holds the weight's offset from one.  `name` is the
+    tensor's local name (file name = prefix + name)."""
+    width: int
+    eps: float
+    prefix: str = ""
+    name: str = "weight"
+    kind: str = "rms_norm_one_plus"
+
+
+@dataclass(frozen=True)
 class RopeSpec:
     """Rotary position encoding over the first `rotary_dim` dims of a head.
 
@@ -107,13 +118,77 @@ class AttentionSpec:
 
 
 @dataclass(frozen=True)
+class MixedHeadAttentionSpec:
+    """Causal grouped-query attention without rotation whose softmax weights are mixed across heads.
+
+    Query head h reads key/value head h // (num_heads / num_kv_heads); keys have `head_dim` values a head,
+    values `v_head_dim`.  q and k are each RMS-normed over their whole projection (all heads at once, plain
+    weight, `qk_norm_eps`).  score = scale * q.k - r1_h * ln(1 + r2_h * distance) (`distance_bias`).  Position i
+    sees j <= i when i - j < `window` (None: every key) or j < `keep_first`.  With `sink` a learned number a head
+    joins the softmax's denominator (no key, no value).  With `head_mixing` the weights of the heads are mixed
+    by a [heads, heads] matrix before they meet the values of each head's own key/value head.  With
+    `output_gate` the concatenated heads are multiplied by sigmoid(W_g x) before the output projection.
+    `names`: the local tensor names of (q, k, v, o, q norm, k norm, r1, r2, sink, mixing matrix, gate).
+    """
+    hidden_size: int
+    num_heads: int
+    num_kv_heads: int
+    head_dim: int
+    v_head_dim: int
+    scale: float
+    qk_norm_eps: float
+    window: Optional[int] = None
+    keep_first: int = 0
+    distance_bias: bool = True
+    sink: bool = True
+    head_mixing: bool = True
+    output_gate: bool = True
+    prefix: str = ""
+    kind: str = "mixed_head_attention"
+    page_size: Optional[int] = None
+    names: Tuple[str, ...] = ("q", "k", "v", "o", "q.norm", "k.norm", "r1", "r2", "sink", "talk", "g")
+
+    def __post_init__(self):
+        if self.num_heads <= 0 or self.num_kv_heads <= 0 or self.num_heads % self.num_kv_heads:
+            raise ConfigError(f"attention heads {self.num_heads} must be a positive multiple of key/value heads {self.num_kv_heads}")
+        for what, d in (("key", self.head_dim), ("value", self.v_head_dim)):
+            if d <= 0 or d > 256:
+                raise ConfigError(f"{what} head size {d} unsupported: the attention kernels take head sizes from 1 to 256")
+        if self.window is not None and self.window <= 0:
+            raise ConfigError(f"attention window must be positive, got {self.window}")
+        if self.keep_first < 0:
+            raise ConfigError(f"keep_first must not be negative, got {self.keep_first}")
+        if self.page_size is not None and self.page_size <= 0:
+            raise ConfigError(f"attention page_size must be positive, got {self.page_size}")
+        if len(self.names) != 11:
+            raise ConfigError("names: eleven local tensor names")
+
+    @property
+    def q_dim(self) -> int:
+        return self.num_heads * self.head_dim
+
+    @property
+    def kv_dim(self) -> int:
+        return self.num_kv_heads * self.head_dim
+
+    @property
+    def v_dim(self) -> int:
+        return self.num_kv_heads * self.v_head_dim
+
+    @property
+    def out_dim(self) -> int:
+        return self.num_heads * self.v_head_dim
+
+
+@dataclass(frozen=True)
 class GatedMLPSpec:
-    """down(act(gate(x)) * up(x)); `activation` is "silu"."""
+    """down(act(gate(x)) * up(x)); `activation` is "silu".  `names`: the local tensor names of (gate, up, down)."""
     hidden_size: int
     intermediate_size: int
     activation: str = "silu"
     prefix: str = ""
     kind: str = "gated_mlp"
+    names: Tuple[str, str, str] = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")
 
     def __post_init__(self):
         if self.intermediate_size <= 0:
@@ -127,10 +202,14 @@ class LayerSpec:
     """One block: `block` names the arrangement, `parts` its parts by role.
 
     The "pre_norm" arrangement has the roles mixer_norm, mixer, ffn_norm, ffn
-    and computes x += mixer(mixer_norm(x)); x += ffn(ffn_norm(x)).
+    and computes x += mixer(mixer_norm(x)); x += ffn(ffn_norm(x)).  The "post_norm"
+    arrangement has the same roles and norms after the sum, the sublayers reading x
+    itself: x = mixer_norm(a x + mixer(x)); x = ffn_norm(a x + ffn(x)) with
+    a = `residual_scale`; "post_norm_mixer" is its first half alone.
     """
     parts: Tuple[Tuple[str, object], ...]
     block: str = "pre_norm"
+    residual_scale: float = 1.0
 
     @property
     def kind(self) -> str:
@@ -154,10 +233,13 @@ class LayerRun:
 
 @dataclass(frozen=True)
 class EmbeddingSpec:
+    """x = table[token] * scale; the table is the tensor prefix + name."""
     vocab_size: int
     hidden_size: int
     prefix: str = "model.embed_tokens."
     kind: str = "embedding"
+    scale: float = 1.0
+    name: str = "weight"
 
 
 @dataclass(frozen=True)

@@ -287,6 +287,43 @@ __global__ void gather_rows_kernel(const uint32_t* __restrict__ x, const int32_t
     for (int i = threadIdx.x; i < width; i += blockDim.x) out[dst + i] = x[src + i];
 }
 
+
+// x[t, :] = table[token[t], :] * scale, the product in float32 (an embedding with a scale of its own).
+template <typename TW>
+__global__ void embed_scaled_kernel(const TW* __restrict__ table, const int32_t* __restrict__ tokens,
+                                    float* __restrict__ out, int hidden, float scale) {
+    const size_t t = blockIdx.x;
+    const size_t row = (size_t)tokens[t] * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) out[t * hidden + i] = load_f(table, row + i) * scale;
+}
+
+// The norm AFTER the residual sum: x <- (alpha x + delta) * rsqrt(mean((alpha x + delta)^2) + eps) * w, written back
+// to the float32 residual stream and, where `rows` is given, once more in the type the next products read.  `delta`
+// may come in slabs that are added in order behind alpha x.  One workgroup a row; the sum lies in x between the passes
+// (every thread reads back what it wrote itself), so any width runs; all of it float32, and the order of a row's
+// additions is fixed by the workgroup's size alone.
+template <typename TD, typename TO>
+__global__ void __launch_bounds__(256) scaled_add_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__ delta,
+                                                                 const float* __restrict__ weight, TO* __restrict__ rows,
+                                                                 int width, float eps, float alpha, int parts, size_t part_stride) {
+    __shared__ float scratch[16];
+    const size_t base = (size_t)blockIdx.x * width;
+    float ss = 0.0f;
+    for (int i = threadIdx.x; i < width; i += 256) {
+        float v = x[base + i] * alpha;
+        for (int p = 0; p < parts; ++p) v += load_f(delta, p * part_stride + base + i);
+        x[base + i] = v;
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float scale = 1.0f / sqrtf(ss / (float)width + eps);
+    for (int i = threadIdx.x; i < width; i += 256) {
+        const float y = x[base + i] * scale * weight[i];
+        x[base + i] = y;
+        if (rows != nullptr) store_f(rows, base + i, y);
+    }
+}
+
 template <typename TD, typename TO>
 static void launch_rmsnorm(float* x, const void* delta, const float* weight, void* out, int rows, int width, float eps,
                            int parts, hipStream_t stream) {
@@ -326,6 +363,34 @@ int kipp_embed(const void* table, int table_dtype, const int32_t* tokens, float*
         hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)table, tokens, out, hidden);
     else
         hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, (const float*)table, tokens, out, hidden);
+    return KIPP_LAUNCH_CHECK();
+}
+
+int kipp_embed_scaled(const void* table, int table_dtype, const int32_t* tokens, float* out,
+                      int n_tokens, int hidden, float scale, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    dim3 grid(n_tokens), block(256);
+    if (table_dtype == KIPP_BF16)
+        hipLaunchKernelGGL(embed_scaled_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)table, tokens, out, hidden, scale);
+    else
+        hipLaunchKernelGGL(embed_scaled_kernel<float>, grid, block, 0, stream, (const float*)table, tokens, out, hidden, scale);
+    return KIPP_LAUNCH_CHECK();
+}
+
+// x = norm(alpha x + delta) in place; `rows` (may be null) receives the same rows in `rows_dtype`; `delta` may be null
+// (parts 0).
+int kipp_scaled_add_rmsnorm(float* x, const void* delta, int delta_dtype, int parts, const float* weight, void* rows,
+                            int rows_dtype, int n_rows, int width, float eps, float alpha, hipStream_t stream) {
+    if (n_rows <= 0 || width <= 0) return 0;
+    if (parts < 0 || (parts > 0 && delta == nullptr)) return -1;
+    const size_t stride = (size_t)n_rows * width;
+#define KIPP_PN(TD, TO) hipLaunchKernelGGL((scaled_add_rmsnorm_kernel<TD, TO>), dim3(n_rows), dim3(256), 0, stream, x, (const TD*)delta, weight, (TO*)rows, width, eps, alpha, parts, stride)
+    if (delta_dtype == KIPP_BF16) {
+        if (rows_dtype == KIPP_BF16) KIPP_PN(bf16_t, bf16_t); else KIPP_PN(bf16_t, float);
+    } else {
+        if (rows_dtype == KIPP_BF16) KIPP_PN(float, bf16_t); else KIPP_PN(float, float);
+    }
+#undef KIPP_PN
     return KIPP_LAUNCH_CHECK();
 }
 

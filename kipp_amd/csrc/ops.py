@@ -97,6 +97,37 @@ def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> torch
     return out
 
 
+def embed_scaled(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor, scale: float) -> torch.Tensor:
+    """out[t] = table[tokens[t]] * scale, in float32."""
+    _dev(table, tokens, out)
+    _i32(tokens, "tokens")
+    n, hidden = out.shape
+    _need(table.dim() == 2 and table.shape[1] == hidden, "embed: table width differs from output width")
+    _need(tokens.numel() == n and out.dtype == torch.float32, "embed: one float32 output row per token")
+    fn = _fn("elementwise", "kipp_embed_scaled", [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_ptr])
+    _check(fn(_ptr(table), _code(table), _ptr(tokens), _ptr(out), n, hidden, float(scale), _stream()), "embed_scaled")
+    return out
+
+
+def scaled_add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], alpha: float, weight: torch.Tensor, eps: float,
+                       rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x <- rmsnorm(alpha * x + delta) * weight in place (float32); `rows`, if given, receives the same rows in its
+    own type.  `delta` is [rows, width], or slabs [parts, rows, width] that are added in order, or None."""
+    _dev(x, weight, delta, rows)
+    n, width = x.shape
+    _need(x.dtype == torch.float32 and weight.dtype == torch.float32, "scaled_add_rmsnorm: x and weight are float32")
+    _need(weight.numel() == width and (rows is None or rows.shape == x.shape), "scaled_add_rmsnorm: shapes differ")
+    parts = 0
+    if delta is not None:
+        _need(tuple(delta.shape[-2:]) == tuple(x.shape) and delta.dim() in (2, 3), "scaled_add_rmsnorm: delta shape differs from x")
+        parts = delta.shape[0] if delta.dim() == 3 else 1
+    fn = _fn("elementwise", "kipp_scaled_add_rmsnorm",
+             [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_float, _c_ptr])
+    _check(fn(_ptr(x), _ptr(delta), _code(delta) if delta is not None else F32, parts, _ptr(weight), _ptr(rows),
+              _code(rows) if rows is not None else F32, n, width, float(eps), float(alpha), _stream()), "scaled_add_rmsnorm")
+    return x
+
+
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
             delta: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out = rmsnorm(x [+ delta]) * weight; with `delta`, x += delta in place.
@@ -275,6 +306,87 @@ def _attn_common(q, k_cache, v_cache, out, n_q, n_kv, head_dim, what):
     _need(head_dim % 16 == 0 and 0 < head_dim <= 256 and n_q % n_kv == 0, f"{what}: head size or head counts refused")
     page = k_cache.shape[2]
     _need(page > 0 and page & (page - 1) == 0, f"{what}: the page size must be a power of two (the generic kernel takes any)")
+
+
+# --------------------------------------------------------------------------- attention with mixed heads
+
+def _slabs(t: torch.Tensor, what: str):
+    """(parts, rows, width) of a float32 product that may come in slabs [parts, rows, width]."""
+    _need(t.dtype == torch.float32 and t.dim() in (2, 3), f"{what}: a float32 product [rows, width] or its slabs")
+    return (1,) + tuple(t.shape) if t.dim() == 2 else tuple(t.shape)
+
+
+def mixed_prepare(proj: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                  positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
+                  n_q: int, n_kv: int, d: int, dv: int, q_weight: torch.Tensor, k_weight: torch.Tensor, eps: float,
+                  write_kv: bool = True) -> torch.Tensor:
+    """From a step's projections `proj` (float32 [tokens, >= n_q d + n_kv d + n_kv dv], columns q | k | v | ..., or
+    slabs of it): q and k RMS-normed over their whole width with plain weights, q kept in `q_out`, k and v
+    written into the pages of their positions."""
+    _dev(proj, q_out, k_cache, v_cache, positions, seq_of_token, block_table, q_weight, k_weight)
+    for t, name in ((positions, "positions"), (seq_of_token, "seq_of_token"), (block_table, "block_table")):
+        _i32(t, name)
+    parts, n, stride = _slabs(proj, "mixed_prepare")
+    _need(stride >= n_q * d + n_kv * d + n_kv * dv, "mixed_prepare: the projections are narrower than q, k and v")
+    _need(q_out.shape == (n, n_q * d) and positions.numel() == n and seq_of_token.numel() == n, "mixed_prepare: one row a token")
+    _need(q_weight.dtype == torch.float32 and k_weight.dtype == torch.float32 and q_weight.numel() == n_q * d
+          and k_weight.numel() == n_kv * d, "mixed_prepare: float32 norm weights over the whole projections")
+    _need(k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.shape[:3] == v_cache.shape[:3] and k_cache.shape[1] == n_kv
+          and k_cache.shape[3] == d and v_cache.shape[3] == dv and k_cache.dtype == v_cache.dtype,
+          "mixed_prepare: caches must be [pages, n_kv, page, d] and [pages, n_kv, page, dv]")
+    _need(block_table.dim() == 2, "mixed_prepare: block_table is [sequences, blocks]")
+    fn = _fn("attention_mixed", "kipp_mixed_prepare",
+             [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int,
+              _c_ptr, _c_ptr, _c_ptr, _c_int] + [_c_int] * 7 + [_c_ptr])
+    _check(fn(_ptr(proj), parts, stride, n_q * d, n_q * d + n_kv * d, _ptr(q_weight), _ptr(k_weight), float(eps),
+              _ptr(q_out), _code(q_out), _ptr(k_cache), _ptr(v_cache), _code(k_cache), _ptr(positions), _ptr(seq_of_token),
+              _ptr(block_table), block_table.shape[1], n, n_q, n_kv, d, dv, k_cache.shape[2], int(write_kv), _stream()),
+           "mixed_prepare")
+    return q_out
+
+
+def _mixed_common(q, k_cache, v_cache, out, gate, gate_at, n_q, n_kv, d, dv, r1, r2, sink, mix, what):
+    n = q.shape[0]
+    _need(q.shape == (n, n_q * d) and out.shape == (n, n_q * dv), f"{what}: q is [tokens, n_q d], out [tokens, n_q dv]")
+    _need(k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.shape[:3] == v_cache.shape[:3] and k_cache.shape[1] == n_kv
+          and k_cache.shape[3] == d and v_cache.shape[3] == dv, f"{what}: caches must be [pages, n_kv, page, d] and [pages, n_kv, page, dv]")
+    _need(n_kv > 0 and n_q % n_kv == 0, f"{what}: query heads must be a multiple of key/value heads")
+    for t, size, name in ((r1, n_q, "r1"), (r2, n_q, "r2"), (sink, n_q, "sink"), (mix, n_q * n_q, "mix")):
+        _need(t is None or (t.dtype == torch.float32 and t.numel() == size), f"{what}: {name} must be float32 with {size} numbers")
+    _need((r1 is None) == (r2 is None), f"{what}: the distance bias needs both of its numbers a head")
+    gate_parts, gate_stride = 0, 0
+    if gate is not None:
+        gate_parts, rows, gate_stride = _slabs(gate, what)
+        _need(rows == n and 0 <= gate_at and gate_at + n_q * dv <= gate_stride, f"{what}: the gate's columns lie outside its rows")
+    return n, gate_parts, gate_stride
+
+
+def mixed_attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
+                          positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
+                          n_q: int, n_kv: int, d: int, dv: int, scale: float, window: int, keep_first: int,
+                          r1: Optional[torch.Tensor], r2: Optional[torch.Tensor], sink: Optional[torch.Tensor],
+                          mix: Optional[torch.Tensor], gate: Optional[torch.Tensor] = None, gate_at: int = 0) -> torch.Tensor:
+    """Attention with a distance bias, kept first keys beside a window, a sink in the softmax, heads mixed after the
+    softmax and an output gate, for every token of a step (one workgroup a token; float32 or bfloat16 storage, float32
+    arithmetic).  `gate`: a float32 product (or its slabs) whose columns from `gate_at` on hold the gate's logits."""
+    _dev(q, k_cache, v_cache, out, positions, seq_of_token, block_table, r1, r2, sink, mix, gate)
+    for t, name in ((positions, "positions"), (seq_of_token, "seq_of_token"), (block_table, "block_table")):
+        _i32(t, name)
+    n, gate_parts, gate_stride = _mixed_common(q, k_cache, v_cache, out, gate, gate_at, n_q, n_kv, d, dv, r1, r2, sink, mix,
+                                               "mixed_attention_plain")
+    _need(0 < d <= 256 and 0 < dv <= 256 and n_q <= 64, "mixed_attention_plain: head sizes up to 256, up to 64 heads")
+    lib = "attention_mixed"
+    lds = _fn(lib, "kipp_mixed_attention_lds_bytes", [_c_int, _c_int])(n_q, d)
+    _need(lds <= 64 * 1024, f"mixed_attention_plain: {n_q} heads of {d} need {lds} bytes of LDS, more than 65,536")
+    fn = _fn(lib, "kipp_mixed_attention",
+             [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
+              _c_ptr, _c_ptr, _c_ptr, _c_ptr] + [_c_int] * 6 + [_c_float, _c_int, _c_int, _c_ptr])
+    gate_ptr = gate.data_ptr() + 4 * gate_at if gate is not None else None
+    _check(fn(_ptr(q), _code(q), _ptr(k_cache), _ptr(v_cache), _code(k_cache), _ptr(out), _code(out), gate_ptr, gate_stride,
+              gate_parts, _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1],
+              _ptr(r1), _ptr(r2), _ptr(sink), _ptr(mix), n, n_q, n_kv, d, dv, k_cache.shape[2], float(scale),
+              int(window), int(keep_first), _stream()), "mixed_attention_plain")
+    return out
 
 
 PREFILL_MAX_BLOCKS = 4096   # table entries of one sequence the prefill kernel stages in LDS

@@ -15,7 +15,7 @@ from typing import Callable, Dict, Tuple
 class ParamSpec:
     """A tensor a part needs.  kind "float": a matrix or vector of reals;
     "int": an integer table (kept as int32).  `init` is how the random-weights
-    mode fills it: ("normal", std) or ("one_plus_normal", std)."""
+    mode fills it: ("normal", std), ("one_plus_normal", std) or ("abs_normal", std)."""
     shape: Tuple[int, ...]
     kind: str = "float"
     init: Tuple[str, float] = ("normal", 0.02)

@@ -49,3 +49,48 @@ class PreNormBlock:
         if not getattr(ffn, "takes_scaled_rows", False):
             h = rt.rows_of(h)
         return x, ffn.forward(h, batch)
+
+
+@register("block", "post_norm")
+class PostNormBlock:
+    """The norm after the sum: x = mixer_norm(a x + mixer(x)); x = ffn_norm(a x + ffn(x)), a = the layer's
+    `residual_scale`.  The sublayers read x itself, so the float32 residual stream is what the norms write; under
+    bfloat16 the norm's kernel writes the same rows once more in bfloat16 for the products that follow (kept in the
+    step's cache for the next block of this kind, which would otherwise cast x again).  Nothing is left pending."""
+
+    roles = (("mixer_norm", "norm"), ("mixer", "mixer"), ("ffn_norm", "norm"), ("ffn", "feed_forward"))
+
+    def __init__(self, layer_spec, runtime):
+        self.rt = runtime
+        self.alpha = float(layer_spec.residual_scale)
+        self.parts = {role: build_part(cat, layer_spec.part(role), runtime) for role, cat in self.roles}
+        self.mixer = self.parts["mixer"]
+        self.graph_safe = all(getattr(part, "graph_safe", False) for part in self.parts.values())
+
+    def _rows(self, x, batch):
+        """x in the type the products read."""
+        import torch
+        if self.rt.act_dtype == torch.float32:
+            return x
+        kept = batch.step_cache.get("residual_rows")
+        if kept is not None and kept[0] is x:
+            return kept[1]
+        return self.rt.ops.cast(x, self.rt.empty(x.shape, self.rt.act_dtype))
+
+    def forward(self, x, pending, batch, cache, state):
+        rt = self.rt
+        if pending is not None:
+            rt.ops.residual_add(x, rt.settle(pending))
+        h = self._rows(x, batch)
+        h = self.parts["mixer_norm"].post_forward(x, self.mixer.forward(h, batch, cache, state), self.alpha, rt.act_dtype)
+        if "ffn" in self.parts:
+            h = self.parts["ffn_norm"].post_forward(x, self.parts["ffn"].forward(h, batch), self.alpha, rt.act_dtype)
+        batch.step_cache["residual_rows"] = (x, h)
+        return x, None
+
+
+@register("block", "post_norm_mixer")
+class PostNormMixerBlock(PostNormBlock):
+    """The first half of the post-norm arrangement alone: a layer without a feed-forward."""
+
+    roles = (("mixer_norm", "norm"), ("mixer", "mixer"))

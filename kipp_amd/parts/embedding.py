@@ -6,7 +6,8 @@ from .base import ParamSpec, register
 
 @register("embedding", "embedding")
 class Embedding:
-    """x[t] = E[token_t], widened to float32, no scaling (/root/reference/src/kipp.c:2579-2585)."""
+    """x[t] = E[token_t], widened to float32 (/root/reference/src/kipp.c:2579-2585), times the spec's `scale`
+    where that is not 1 (the product in float32).  The table is the tensor `spec.name`."""
 
     graph_safe = True   # forward launches kernels only: no host reads, no data-dependent launches
 
@@ -17,13 +18,16 @@ class Embedding:
 
     @staticmethod
     def params(spec):
-        return {"weight": ParamSpec((spec.vocab_size, spec.hidden_size))}
+        return {getattr(spec, "name", "weight"): ParamSpec((spec.vocab_size, spec.hidden_size))}
 
     def load(self, tensors):
-        self.weight = tensors["weight"]
+        self.weight = tensors[getattr(self.spec, "name", "weight")]
 
     def forward(self, tokens):
         import torch
+        scale = float(getattr(self.spec, "scale", 1.0))
+        if scale != 1.0:
+            return self.rt.ops.embed_scaled(self.weight, tokens, self.rt.empty((tokens.numel(), self.spec.hidden_size), torch.float32), scale)
         return self.rt.ops.embed(self.weight, tokens, self.rt.empty((tokens.numel(), self.spec.hidden_size), torch.float32))
 
 

@@ -30,18 +30,20 @@ class GatedMLP:
 
     @staticmethod
     def params(spec):
+        gate, up, down = spec.names
         return {
-            "gate_proj.weight": ParamSpec((spec.intermediate_size, spec.hidden_size)),
-            "up_proj.weight": ParamSpec((spec.intermediate_size, spec.hidden_size)),
-            "down_proj.weight": ParamSpec((spec.hidden_size, spec.intermediate_size)),
+            gate: ParamSpec((spec.intermediate_size, spec.hidden_size)),
+            up: ParamSpec((spec.intermediate_size, spec.hidden_size)),
+            down: ParamSpec((spec.hidden_size, spec.intermediate_size)),
         }
 
     def load(self, tensors):
-        g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
+        gate, up, down = self.spec.names
+        g, u = tensors[gate], tensors[up]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
         self.w_gate_up = self.rt.weight(torch.cat([g, u], dim=0).contiguous(), gate_up=True)
-        self.w_down = self.rt.weight(tensors["down_proj.weight"])
+        self.w_down = self.rt.weight(tensors[down])
 
     def forward(self, x, batch=None):
         rt = self.rt

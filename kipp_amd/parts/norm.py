@@ -4,6 +4,10 @@
     load(tensors)                       tensors by local name, already on the device
     forward(x, out_dtype) -> y          x float32 [rows, width]
     add_forward(x, delta, out_dtype)    x += delta in place, then y = norm(x)
+    post_forward(x, delta, alpha, rows_dtype) -> rows
+                                        x = norm(alpha x + delta) in place (the norm after the sum, whose result IS
+                                        the residual stream); `rows`: the same in `rows_dtype` for the next products
+                                        (x itself where that is float32).  Optional: what a post-norm block needs.
 
 A norm with `fuses_products = True` also takes a delta that `Runtime.linear(...,
 defer=True)` has not launched yet and may return `ScaledRows` (its rows without
@@ -50,3 +54,27 @@ class RMSNorm:
                 return fused
             delta = delta.run()
         return self.rt.ops.rmsnorm(x, self.weight, self.spec.eps, self.rt.empty(x.shape, out_dtype), delta=delta)
+
+    def post_forward(self, x, delta, alpha, rows_dtype):
+        import torch
+        delta = self.rt.settle(delta)
+        rows = None if rows_dtype == torch.float32 else self.rt.empty(x.shape, rows_dtype)
+        self.rt.ops.scaled_add_rmsnorm(x, delta, alpha, self.weight, self.spec.eps, rows)
+        return x if rows is None else rows
+
+
+@register("norm", "rms_norm_one_plus")
+class OnePlusRMSNorm(RMSNorm):
+    """y = x * rsqrt(mean(x^2) + eps) * (1 + w): the tensor holds the offset of the weight from one.  The one is added once, at
+    load, in float32; from there on it is the plain norm and rides on the same kernels."""
+
+    @staticmethod
+    def params(spec):
+        return {spec.name: ParamSpec((spec.width,), "float", ("normal", 0.05))}
+
+    @staticmethod
+    def placement(spec):
+        return {spec.name: "float32"}
+
+    def load(self, tensors):
+        self.weight = (tensors[self.spec.name].float() + 1.0).contiguous()

@@ -3,7 +3,8 @@ configuration and a seed.
 
 Each tensor has its own stream, seeded by (seed, tensor name), so the values
 do not depend on the order of creation.  Matrices and the embedding are
-N(0, std), norm weights 1 + N(0, std), with the std that the part declares.
+N(0, std), norm weights 1 + N(0, std), numbers that must not be negative |N(0, std)|, with the std that the
+part declares.
 Values are drawn in float32 and stored as `dtype` (bfloat16: round to nearest
 even).
 """
@@ -36,6 +37,8 @@ def random_tensor(seed: int, name: str, spec: ParamSpec, dtype: torch.dtype = to
     t = torch.empty(spec.shape, dtype=torch.float32, device=device).normal_(0.0, std, generator=gen)
     if how == "one_plus_normal":
         t += 1.0
+    elif how == "abs_normal":
+        t.abs_()
     elif how != "normal":
         raise ValueError(f"unknown init {how!r} for {name}")
     return t.to(dtype)
