@@ -8,6 +8,8 @@
 //   p'_h = sum_g mix[h, g] p_g;  o_h(i) = sum_j p'_h(i, j) v_c(j);  out = o * sigmoid(gate)
 //
 // Keys and values have sizes of their own (d and dv).  Scores, softmax, the mixing and all sums are float32.
+// Keys lie in the cache as [page][kv head][slot][d]; values transposed inside a page, [page][kv head][dv][slot]
+// (the same bytes a page: the matrix-core form reads eight keys of one value column as sixteen contiguous bytes).
 //
 // Two kernels: `mixed_prepare_kernel` norms q and k of every token of a step, keeps q and writes k and v into
 // their pages; `mixed_attention_kernel` (this file's plain form: one workgroup a token, the float32 path's kernel
@@ -26,7 +28,7 @@
 #define MIXED_HPW (MIXED_MAX_HEADS / MIXED_WAVES)      // heads a wave carries at most
 
 // proj [n, stride] float32 holds a token's projections: q at column 0 (n_q * d), k at `k_at` (n_kv * d), v at `v_at`
-// (n_kv * dv).  One workgroup a token.
+// (n_kv * dv).  One workgroup a token.  Values are written transposed inside their page.
 template <typename TQ, typename TC>
 __global__ void __launch_bounds__(MIXED_THREADS) mixed_prepare_kernel(
     const float* __restrict__ proj, int parts, size_t part_stride, int stride, int k_at, int v_at,
@@ -72,7 +74,7 @@ __global__ void __launch_bounds__(MIXED_THREADS) mixed_prepare_kernel(
         float v = 0.0f;
         for (int p = 0; p < parts; ++p) v += row[p * part_stride + v_at + e];
         const int g = e / dv, i = e - g * dv;
-        store_f(v_cache, (((size_t)page_id * n_kv + g) * page + slot) * dv + i, v);
+        store_f(v_cache, (((size_t)page_id * n_kv + g) * dv + i) * page + slot, v);      // transposed inside the page
     }
 }
 
@@ -93,7 +95,8 @@ __global__ void __launch_bounds__(MIXED_THREADS) mixed_attention_kernel(
     float* pm_s = p_s + (size_t)n_q * KIPP_WAVE;        // [n_q][64]: the weights after the heads are mixed
     float* m_s = pm_s + (size_t)n_q * KIPP_WAVE;        // [n_q]
     float* l_s = m_s + n_q;                             // [n_q]
-    long long* page_s = (long long*)(l_s + n_q + ((n_q & 1) ? 1 : 0));   // [64]: page id * n_kv * page + slot, or -1
+    long long* page_s = (long long*)(l_s + n_q + ((n_q & 1) ? 1 : 0));   // [64]: page id * n_kv of the tile's keys
+    int* slot_s = (int*)(page_s + KIPP_WAVE);                            // [64]: their slots in the page
     const int wave = threadIdx.x / KIPP_WAVE;
     const int lane = threadIdx.x & (KIPP_WAVE - 1);
     const int t = blockIdx.x;
@@ -147,13 +150,16 @@ __global__ void __launch_bounds__(MIXED_THREADS) mixed_attention_kernel(
         for (int s0 = (from / KIPP_WAVE) * KIPP_WAVE; s0 <= to; s0 += KIPP_WAVE) {
             const int s = s0 + lane;
             const bool valid = s >= from && s <= to;
-            const long long at = valid ? ((long long)table[s / page] * n_kv * page + s % page) : -1;
-            if (wave == 0) page_s[lane] = at;
+            const long long at = valid ? (long long)table[s / page] * n_kv : 0;
+            if (wave == 0) {
+                page_s[lane] = at;
+                slot_s[lane] = s % page;
+            }
             for (int h = wave; h < n_q; h += MIXED_WAVES) {
                 const int c = h / group;
                 float p = 0.0f;
                 if (valid) {
-                    const TC* k_row = k_cache + ((size_t)at + (size_t)c * page) * d;
+                    const TC* k_row = k_cache + (((size_t)at + c) * page + s % page) * d;
                     float dot = 0.0f;
                     for (int e = 0; e < d; ++e) dot = fmaf(q_s[h * d + e], load_f(k_row, e), dot);
                     const float a = r1 != nullptr ? r1[h] : 0.0f, b = r2 != nullptr ? r2[h] : 0.0f;
@@ -184,7 +190,7 @@ __global__ void __launch_bounds__(MIXED_THREADS) mixed_attention_kernel(
                         if (e < dv) {
                             float a = acc[i][cc];
                             for (int j = j_lo; j < j_hi; ++j)
-                                a = fmaf(w_s[h * KIPP_WAVE + j], load_f(v_cache, ((size_t)page_s[j] + (size_t)c * page) * dv + e), a);
+                                a = fmaf(w_s[h * KIPP_WAVE + j], load_f(v_cache, (((size_t)page_s[j] + c) * dv + e) * page + slot_s[j]), a);
                             acc[i][cc] = a;
                         }
                     }
@@ -237,7 +243,7 @@ int kipp_mixed_prepare(const float* proj, int parts, int stride, int k_at, int v
 }
 
 int kipp_mixed_attention_lds_bytes(int n_q, int d) {
-    return (int)(((size_t)n_q * d + 2 * (size_t)n_q * KIPP_WAVE + 2 * n_q + (n_q & 1)) * 4 + KIPP_WAVE * 8);
+    return (int)(((size_t)n_q * d + 2 * (size_t)n_q * KIPP_WAVE + 2 * n_q + (n_q & 1)) * 4 + KIPP_WAVE * 12);
 }
 
 int kipp_mixed_attention(const void* q, int q_dtype, const void* k_cache, const void* v_cache, int cache_dtype, void* out, int out_dtype,

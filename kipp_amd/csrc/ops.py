@@ -389,6 +389,71 @@ def mixed_attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
     return out
 
 
+MIXED_ROWS = 16         # query rows of a tile of the matrix-core form
+MIXED_KEYS = 32         # keys it takes at a time
+MIXED_WAVES = 8
+
+
+def mixed_attention_defines(n_q: int, d: int, dv: int) -> dict:
+    """The build of attention_mixed_mfma.hip that takes these sizes."""
+    return {"HEAD_DIM": d, "V_DIM": dv, "HPW": -(-n_q // MIXED_WAVES)}
+
+
+def mixed_attention_fast_ok(n_q: int, d: int, dv: int, page: int) -> bool:
+    """Whether the matrix-core form takes this geometry: key size a multiple of 32, value size a multiple of 16,
+    up to 32 heads whose sums fit a wave's registers, pages of a multiple of 16 keys."""
+    hpw = -(-n_q // MIXED_WAVES)
+    return d % 32 == 0 and 0 < d <= 256 and dv % 16 == 0 and 0 < dv <= 256 and 0 < n_q <= 32 and hpw * (dv // 16) <= 32 \
+        and page > 0 and page % 16 == 0
+
+
+def mixed_attention_workspace(n_items: int, n_rows: int, n_q: int, dv: int, max_splits: int, device) -> tuple:
+    """(statistics of every item, partial sums of the rows whose keys are cut into runs or None)."""
+    stats = torch.empty((n_items, n_q, MIXED_ROWS, 2), dtype=torch.float32, device=device)
+    partial = torch.empty((max_splits, n_rows, n_q * dv), dtype=torch.float32, device=device) if max_splits > 1 else None
+    return stats, partial
+
+
+def mixed_attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
+                         items: tuple, n_items: int, row_splits: Optional[torch.Tensor], max_splits: int,
+                         q_start: torch.Tensor, q_len: torch.Tensor, ctx_len: torch.Tensor, block_table: torch.Tensor,
+                         n_q: int, n_kv: int, d: int, dv: int, scale: float, window: int, keep_first: int,
+                         r1: Optional[torch.Tensor], r2: Optional[torch.Tensor], sink: Optional[torch.Tensor],
+                         mix: Optional[torch.Tensor], workspace: tuple, gate: Optional[torch.Tensor] = None,
+                         gate_at: int = 0) -> torch.Tensor:
+    """The same attention on the matrix cores (bfloat16).  `items`: four int32 tensors [n_items] (entry, first row of
+    the tile within the entry, which run of the tile's keys, runs of the tile; a tile's items are consecutive);
+    `row_splits` [rows]: the runs of each row's tile (needed when `max_splits` > 1); `workspace` from
+    `mixed_attention_workspace`.  The kernels take every length from the device (`q_len`, `ctx_len`), so an item
+    list made for longer contexts than the step's stays valid."""
+    stats, partial = workspace
+    _dev(q, k_cache, v_cache, out, *items, row_splits, q_start, q_len, ctx_len, block_table, r1, r2, sink, mix, gate, stats, partial)
+    for t, name in ((q_start, "q_start"), (q_len, "q_len"), (ctx_len, "ctx_len"), (block_table, "block_table")) \
+            + tuple((t, "items") for t in items) + (((row_splits, "row_splits"),) if row_splits is not None else ()):
+        _i32(t, name)
+    n, gate_parts, gate_stride = _mixed_common(q, k_cache, v_cache, out, gate, gate_at, n_q, n_kv, d, dv, r1, r2, sink, mix,
+                                               "mixed_attention_mfma")
+    _need(all(t.dtype == torch.bfloat16 for t in (q, k_cache, v_cache, out)), "mixed_attention_mfma: bfloat16 queries, caches and output")
+    _need(mixed_attention_fast_ok(n_q, d, dv, k_cache.shape[2]), "mixed_attention_mfma: sizes refused (the plain form takes them)")
+    _need(len(items) == 4 and all(t.numel() >= n_items for t in items) and n_items > 0, "mixed_attention_mfma: four lists of n_items")
+    _need(stats.numel() >= n_items * n_q * MIXED_ROWS * 2, "mixed_attention_mfma: the statistics' workspace is too small")
+    _need(max_splits == 1 or (partial is not None and partial.numel() >= max_splits * n * n_q * dv and row_splits is not None
+                              and row_splits.numel() >= n), "mixed_attention_mfma: cut keys need partial sums and the rows' runs")
+    entries = q_start.numel()
+    _need(q_len.numel() == entries and ctx_len.numel() == entries and block_table.dim() == 2 and block_table.shape[0] >= entries,
+          "mixed_attention_mfma: one q_start, q_len, ctx_len and table row an entry")
+    fn = _fn("attention_mixed_mfma", "kipp_mixed_attention_mfma",
+             [_c_ptr] * 5 + [_c_int, _c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr, _c_int] + [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 6
+             + [_c_int] * 6 + [_c_float, _c_int, _c_int, _c_ptr], mixed_attention_defines(n_q, d, dv))
+    gate_ptr = gate.data_ptr() + 4 * gate_at if gate is not None else None
+    _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), gate_ptr, gate_stride, gate_parts,
+              _ptr(items[0]), _ptr(items[1]), _ptr(items[2]), _ptr(items[3]), n_items, _ptr(row_splits), max_splits,
+              _ptr(q_start), _ptr(q_len), _ptr(ctx_len), _ptr(block_table), block_table.shape[1],
+              _ptr(r1), _ptr(r2), _ptr(sink), _ptr(mix), _ptr(stats), _ptr(partial),
+              n, n_q, n_kv, d, dv, k_cache.shape[2], float(scale), int(window), int(keep_first), _stream()), "mixed_attention_mfma")
+    return out
+
+
 PREFILL_MAX_BLOCKS = 4096   # table entries of one sequence the prefill kernel stages in LDS
 
 

@@ -63,7 +63,13 @@ class MixedHeadAttention:
 
     @staticmethod
     def variants(spec, dtype):
-        return [("attention_mixed", None)]
+        """The plain kernels, and under bfloat16 the build of the matrix-core form for these sizes where it takes them
+        (any page size that it takes: the engine's is not known here)."""
+        from ..csrc import ops
+        out = [("attention_mixed", None)]
+        if dtype == "bfloat16" and ops.mixed_attention_fast_ok(spec.num_heads, spec.head_dim, spec.v_head_dim, spec.page_size or 16):
+            out.append(("attention_mixed_mfma", ops.mixed_attention_defines(spec.num_heads, spec.head_dim, spec.v_head_dim)))
+        return out
 
     def load(self, tensors):
         n, s = self._names(self.spec), self.spec
@@ -103,8 +109,56 @@ class MixedHeadAttention:
                               self.q_norm, self.k_norm, s.qk_norm_eps, write_kv=cache.writable)
         out = rt.empty((n, s.out_dim), rt.act_dtype)
         gate_at = s.q_dim + s.kv_dim + s.v_dim
+        if rt.dtype == "bfloat16" and getattr(rt, "mixed_attention_fast", True) \
+                and ops.mixed_attention_fast_ok(s.num_heads, s.head_dim, s.v_head_dim, cache.page_size):
+            items, n_items, row_splits, max_splits, workspace = self._work(batch)
+            ops.mixed_attention_mfma(q, cache.k, cache.v, out, items, n_items, row_splits, max_splits,
+                                     batch.q_start, batch.q_len, batch.ctx_len, table,
+                                     s.num_heads, s.num_kv_heads, s.head_dim, s.v_head_dim, s.scale, s.window or 0,
+                                     s.keep_first, self.r1, self.r2, self.sink, self.mix, workspace,
+                                     gate=proj if s.output_gate else None, gate_at=gate_at)
+            return rt.linear(out, self.w_o, slabs=True, defer=True)
+        if rt.dtype == "bfloat16":
+            rt.generic_attention_launches += 1      # the slow kernel class: a measurement must know it ran
         ops.mixed_attention_plain(q, cache.k, cache.v, out, batch.positions, batch.seq_of_token, table,
                                   s.num_heads, s.num_kv_heads, s.head_dim, s.v_head_dim, s.scale, s.window or 0,
                                   s.keep_first, self.r1, self.r2, self.sink, self.mix,
                                   gate=proj if s.output_gate else None, gate_at=gate_at)
         return rt.linear(out, self.w_o, slabs=True, defer=True)
+
+    def _work(self, batch):
+        """The item list of the matrix-core form: every entry's rows in tiles of 16, and where the tiles alone are too
+        few workgroups to fill the GPU, each tile's keys in several runs (at least 128 keys a run, at most 16 runs).
+        Made by the first layer of a geometry and kept while the batch object lives: a recorded step keeps its own,
+        made for the longest context of its class (the kernels take the true lengths from the device)."""
+        s, ops = self.spec, self.rt.ops
+        key = ("mixed_attention_work", s.num_heads, s.v_head_dim, s.window, s.keep_first)
+        work = batch.host.get(key)
+        if work is None:
+            rows_tile, keys_tile = ops.MIXED_ROWS, ops.MIXED_KEYS
+            window, keep = s.window or 0, s.keep_first
+            tiles = []
+            for e, (n, ctx) in enumerate(zip(batch.host["q_len"], batch.host["ctx_len"])):
+                for row0 in range(0, n, rows_tile):
+                    rows = min(rows_tile, n - row0)
+                    pos0 = ctx - n + row0
+                    lo = max(0, pos0 - window + 1) if window else 0
+                    kept = min(keep, lo) if window else 0
+                    kept_tiles = (kept - 1) // keys_tile + 1 if kept > 0 else 0
+                    first = max(lo // keys_tile, kept_tiles)
+                    tiles.append((e, row0, rows, kept_tiles + (pos0 + rows - 1) // keys_tile - first + 1))
+            want = -(-2 * ops.compute_units(self.rt.device) // len(tiles))
+            entry, row0s, split, nsplits, row_splits = [], [], [], [], []
+            for e, row0, rows, key_tiles in tiles:
+                runs = max(1, min(16, key_tiles // 4, want))
+                entry += [e] * runs
+                row0s += [row0] * runs
+                split += list(range(runs))
+                nsplits += [runs] * runs
+                row_splits += [runs] * rows
+            most = max(nsplits)
+            lists = batch.upload(entry, row0s, split, nsplits, row_splits)
+            space = ops.mixed_attention_workspace(len(entry), batch.n_tokens, s.num_heads, s.v_head_dim, most, self.rt.device)
+            work = (tuple(lists[:4]), len(entry), lists[4], most, space)
+            batch.host[key] = work
+        return work

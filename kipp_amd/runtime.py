@@ -132,6 +132,9 @@ class Runtime:
         # fewer a layer; ordered by device-scope stores, one device-scope counter a head and device-scope loads); False,
         # or KIPP_AMD_DECODE_MERGE=launch, merges them in a launch of its own, which needs no ordering between workgroups
         self.merge_in_kernel = os.environ.get("KIPP_AMD_DECODE_MERGE", "kernel") != "launch"
+        # attention with mixed heads under bfloat16: the matrix-core form where it takes the sizes; False, or
+        # KIPP_AMD_MIXED_ATTENTION=plain, runs the plain kernel (one workgroup a token) everywhere
+        self.mixed_attention_fast = os.environ.get("KIPP_AMD_MIXED_ATTENTION", "mfma") != "plain"
         self.for_a_graph = False    # set around a step of single tokens that is, or is to be, recorded as a HIP graph
         torch.backends.cuda.matmul.allow_tf32 = False
 
