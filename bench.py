@@ -47,7 +47,7 @@ def model_numbers(spec, cache_groups, element_size):
     the cache bytes a token holds (from the cache groups) and the attention flops per (query, key) pair."""
     from kipp_amd.engine.model import model_params
     params = model_params(spec)
-    embedding = spec.embedding.prefix + "weight"
+    embedding = spec.embedding.prefix + getattr(spec.embedding, "name", "weight")
     head = embedding if spec.head.tied else spec.head.prefix + "weight"
 
     def numel(p):
@@ -244,6 +244,87 @@ def long_context_points(model, rt, cfg, numbers, args, weight_bytes, kv_per_toke
     return points, fracs
 
 
+def tobinex_config(qwen: dict, layers: int, window) -> dict:
+    """A Tobinex configuration with the layer sizes of a Qwen3 shape: the same width, heads, head size (keys and values
+    alike), feed-forward and vocabulary; `window` None keeps every key, as the Qwen3 layers do."""
+    heads = qwen["num_attention_heads"]
+    head_dim = qwen.get("head_dim") or qwen["hidden_size"] // heads
+    mixer = {"heads": heads, "kv_heads": qwen["num_key_value_heads"], "dim": head_dim, "vdim": head_dim,
+             "scale": head_dim ** -0.5, "mask": {"size": window, "keep_first": 4} if window else None}
+    return {"architecture": "Tobinex", "vocab": qwen["vocab_size"], "width": qwen["hidden_size"], "embedding": {"scale": 1.0},
+            "norm": {"eps": 1e-6}, "postln_alpha": 1.0, "max_position": 8192,
+            "layers": [{"type": "attention", "mixer": dict(mixer), "mlp": {"kind": "dense", "ff": qwen["intermediate_size"]}}
+                       for _ in range(layers)]}
+
+
+def design_points(config, args, label):
+    """Prefill of one 2,048-token prompt and decode steps at two batch sizes behind such prompts, for one model made
+    with random weights: milliseconds, tokens a second, and what the kernels ran as (recorded steps, library products,
+    attention launches that fell to a plain kernel)."""
+    import torch
+    from kipp_amd.engine import Engine, StepEntry, random_model
+    from kipp_amd.runtime import Runtime
+    rt = Runtime("bfloat16")
+    model = random_model(config, seed=0, runtime=rt)
+    vocab = model.spec.vocab_size
+    batches, page = (8, 64), 16
+    steps, warmup = args.steps, max(args.warmup, 3)
+    room = args.prompt + 2 * (steps + warmup + 2) + 16
+    engine = Engine(model, page_size=page, num_pages=max(batches) * (-(-room // page)) + 4, max_requests=max(batches),
+                    share_prefixes=False, max_position=room + page)
+    out = {}
+    gen = torch.Generator().manual_seed(1)
+    times = []
+    for _ in range(5):
+        toks = torch.randint(0, vocab, (PREFILL_TOKENS,), generator=gen).tolist()
+        torch.cuda.synchronize()
+        start = time.perf_counter()
+        engine.step([StepEntry("prefill", toks, [PREFILL_TOKENS - 1])])
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - start)
+        engine.close("prefill")
+    best = sorted(times[1:])[len(times[1:]) // 2]
+    out["prefill_2048_ms"] = round(best * 1e3, 3)
+    out["prefill_tok_s"] = round(PREFILL_TOKENS / best, 1)
+    log(f"{label}: prefill of {PREFILL_TOKENS} tokens {best * 1e3:.2f} ms")
+    ids = [f"d{i}" for i in range(max(batches))]
+    first = fill(engine, ids, args.prompt, vocab, seed=2)
+    at = args.prompt
+    for b in batches:
+        # every batch size goes on from where the one before stopped: contexts of args.prompt and a few hundred more
+        replays = engine.graphs.replays
+        seconds = decode_run(engine, ids[:b], first, steps, warmup)
+        out[f"decode_b{b}_ms"] = round(seconds / steps * 1e3, 4)
+        out[f"decode_b{b}_tok_s"] = round(b * steps / seconds, 1)
+        out[f"decode_b{b}_replays"] = engine.graphs.replays - replays
+        log(f"{label}: decode batch {b}: {seconds / steps * 1e3:.3f} ms a step, {b * steps / seconds:.0f} tok/s")
+    out["library_products"] = rt.library_products
+    out["plain_attention_launches"] = rt.generic_attention_launches
+    del engine, model
+    torch.cuda.empty_cache()
+    return out
+
+
+def design_bench(args) -> int:
+    """`--design tobinex`: the Tobinex design beside Qwen3 at equal layer sizes (both with every key kept, and Tobinex
+    once more with a window of 1,024 keys behind 4 kept ones), a few layers of each, random weights."""
+    from kipp_amd.config import shape_config
+    layers = args.layers or 4
+    sizes = {}
+    for shape in [s for s in args.design_shapes.split(",") if s]:
+        qwen = shape_config(shape)
+        qwen["num_hidden_layers"] = layers
+        sizes[shape] = {
+            "qwen3": design_points(qwen, args, f"{shape} qwen3"),
+            "tobinex": design_points(tobinex_config(qwen, layers, None), args, f"{shape} tobinex"),
+            "tobinex_window_1024": design_points(tobinex_config(qwen, layers, 1024), args, f"{shape} tobinex, window 1024"),
+        }
+    print(json.dumps({"metric": "prefill and decode of the Tobinex design beside Qwen3 at equal layer sizes (bf16, random weights)",
+                      "design": "tobinex", "layers": layers, "prompt_tokens": args.prompt, "steps": args.steps,
+                      "unit": "ms and tok/s", "n_gpus": 1, "dtype": "bf16", "data": "synthetic", "sizes": sizes}), flush=True)
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -263,10 +344,15 @@ def main():
     ap.add_argument("--no-c-host", action="store_true", help="leave out the points measured through the C host")
     ap.add_argument("--products", choices=["default", "own", "auto", "library"], default="default",
                     help="products of many rows (prompt portions): the runtime's default, our kernel only, the fastest of ours and the library's, the library's")
+    ap.add_argument("--design", choices=["tobinex"], default=None,
+                    help="instead of the default workload: this design beside Qwen3 at equal layer sizes (prefill and decode, a few layers)")
+    ap.add_argument("--design-shapes", default="qwen3-4b,qwen3-8b", help="the Qwen3 shapes whose layer sizes --design takes")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.design:
+        return design_bench(args)
 
     import torch
     from kipp_amd.config import parse_config, shape_config

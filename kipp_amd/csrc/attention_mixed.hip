@@ -78,6 +78,57 @@ __global__ void __launch_bounds__(MIXED_THREADS) mixed_prepare_kernel(
     }
 }
 
+// The same with a token's sums staged in LDS (dynamic, n_q d + n_kv d + n_kv dv floats): the slabs are read once, four
+// at a time, and every value is normed or written from LDS.  Same sums in the same order as the kernel above.
+template <typename TQ, typename TC>
+__global__ void __launch_bounds__(MIXED_THREADS) mixed_prepare_lds_kernel(
+    const float* __restrict__ proj, int parts, size_t part_stride, int stride, int k_at, int v_at,
+    const float* __restrict__ q_weight, const float* __restrict__ k_weight, float eps,
+    TQ* __restrict__ q_out, TC* __restrict__ k_cache, TC* __restrict__ v_cache,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
+    const int32_t* __restrict__ block_table, int max_blocks, int n_q, int n_kv, int d, int dv, int page, int write_kv) {
+    extern __shared__ float sums[];
+    __shared__ float scratch[16];
+    const int t = blockIdx.x;
+    const float* row = proj + (size_t)t * stride;
+    const int q_dim = n_q * d, k_dim = n_kv * d, v_dim = n_kv * dv;
+    const int total = q_dim + k_dim + v_dim;
+    float ss_q = 0.0f, ss_k = 0.0f;
+    for (int e = threadIdx.x; e < total; e += MIXED_THREADS) {
+        const int col = e < q_dim ? e : (e < q_dim + k_dim ? k_at + e - q_dim : v_at + e - q_dim - k_dim);
+        float v = 0.0f;
+        for (int p0 = 0; p0 < parts; p0 += 4) {
+            float part[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) part[u] = p0 + u < parts ? row[(p0 + u) * part_stride + col] : 0.0f;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v += part[u];
+        }
+        sums[e] = v;
+        if (e < q_dim) ss_q = fmaf(v, v, ss_q);
+        else if (e < q_dim + k_dim) ss_k = fmaf(v, v, ss_k);
+    }
+    ss_q = block_sum(ss_q, scratch);
+    ss_k = block_sum(ss_k, scratch);
+    const float scale_q = 1.0f / sqrtf(ss_q / (float)q_dim + eps);
+    const float scale_k = 1.0f / sqrtf(ss_k / (float)k_dim + eps);
+    const int pos = positions[t];
+    const int page_id = write_kv ? block_table[(size_t)seq_of_token[t] * max_blocks + pos / page] : 0;
+    const int slot = pos % page;
+    for (int e = threadIdx.x; e < (write_kv ? total : q_dim); e += MIXED_THREADS) {
+        const float v = sums[e];
+        if (e < q_dim) {
+            store_f(q_out, (size_t)t * q_dim + e, v * scale_q * q_weight[e]);
+        } else if (e < q_dim + k_dim) {
+            const int c = e - q_dim, g = c / d, i = c - g * d;
+            store_f(k_cache, (((size_t)page_id * n_kv + g) * page + slot) * d + i, v * scale_k * k_weight[c]);
+        } else {
+            const int c = e - q_dim - k_dim, g = c / dv, i = c - g * dv;
+            store_f(v_cache, (((size_t)page_id * n_kv + g) * dv + i) * page + slot, v);
+        }
+    }
+}
+
 // One workgroup a token, 4 waves; wave w carries heads w, w + 4, ...  LDS (dynamic): q of every head as float32
 // [n_q][d], the tile's weights [n_q][64] before and after the heads are mixed, the tile's page offsets [64], and
 // every head's maximum and denominator.
@@ -231,10 +282,20 @@ int kipp_mixed_prepare(const float* proj, int parts, int stride, int k_at, int v
     if (n_tokens <= 0) return 0;
     if (parts < 1 || n_q <= 0 || n_kv <= 0 || d <= 0 || dv <= 0 || page <= 0) return -1;
     const size_t part_stride = (size_t)n_tokens * stride;
+    const size_t staged = ((size_t)n_q * d + (size_t)n_kv * d + (size_t)n_kv * dv) * sizeof(float);
 #define KIPP_MP(TQ, TC)                                                                                                    \
-    hipLaunchKernelGGL((mixed_prepare_kernel<TQ, TC>), dim3(n_tokens), dim3(MIXED_THREADS), 0, stream, proj, parts,         \
-                       part_stride, stride, k_at, v_at, q_weight, k_weight, eps, (TQ*)q_out, (TC*)k_cache, (TC*)v_cache,     \
-                       positions, seq_of_token, block_table, max_blocks, n_q, n_kv, d, dv, page, write_kv)
+    do {                                                                                                                   \
+        if (staged <= 48 * 1024)                                                                                           \
+            hipLaunchKernelGGL((mixed_prepare_lds_kernel<TQ, TC>), dim3(n_tokens), dim3(MIXED_THREADS), staged, stream, proj, \
+                               parts, part_stride, stride, k_at, v_at, q_weight, k_weight, eps, (TQ*)q_out, (TC*)k_cache,    \
+                               (TC*)v_cache, positions, seq_of_token, block_table, max_blocks, n_q, n_kv, d, dv, page,      \
+                               write_kv);                                                                                   \
+        else                                                                                                               \
+            hipLaunchKernelGGL((mixed_prepare_kernel<TQ, TC>), dim3(n_tokens), dim3(MIXED_THREADS), 0, stream, proj, parts,  \
+                               part_stride, stride, k_at, v_at, q_weight, k_weight, eps, (TQ*)q_out, (TC*)k_cache,          \
+                               (TC*)v_cache, positions, seq_of_token, block_table, max_blocks, n_q, n_kv, d, dv, page,      \
+                               write_kv);                                                                                   \
+    } while (0)
     if (q_dtype == KIPP_F32 && cache_dtype == KIPP_F32) KIPP_MP(float, float);
     else if (q_dtype == KIPP_BF16 && cache_dtype == KIPP_BF16) KIPP_MP(bf16_t, bf16_t);
     else return -2;

@@ -1,6 +1,7 @@
 // Attention whose softmax weights are mixed across heads, on the matrix cores (bfloat16 storage, float32
 // arithmetic around the products).  The formulas are those at the head of attention_mixed.hip; built for one key
-// size HEAD_DIM (a multiple of 32), one value size V_DIM (a multiple of 16) and HPW heads a wave (up to 8 HPW heads).
+// size HEAD_DIM (a multiple of 32), one value size V_DIM (a multiple of 16) and HPW heads a wave (up to 8 HPW heads);
+// SHARED_KV says that a wave's heads all read one key/value head, whose keys and values it then loads once.
 //
 // Mixing the heads' weights needs every head's FINAL weight of a (query, key) pair in one place, so the softmax
 // cannot be rescaled on the way as flash attention does.  The work is therefore cut into items (a tile of up to 16
@@ -36,6 +37,9 @@
 #endif
 #ifndef HPW
 #define HPW 1
+#endif
+#ifndef SHARED_KV
+#define SHARED_KV 1                     // the HPW heads of a wave read one key/value head (heads a kv head are a multiple of HPW)
 #endif
 
 #define MX_WAVES 8
@@ -102,17 +106,22 @@ __device__ __forceinline__ int key_tile(const Tile& t, int index) {
     return index < t.kept_tiles ? index : t.window_tile0 + index - t.kept_tiles;
 }
 
-// S^T[key][row] of head `h` for the 16 keys from `key0` on: lane l gets keys key0 + 4 (l / 16) + v of row l % 16,
-// already scaled, biased by distance and masked (-inf).  `qf`: the head's query rows as B operands.
-__device__ __forceinline__ void scores16(const MixedGeometry& g, const Tile& t, const bf16_t* __restrict__ k_cache, int h, int key0,
-                                         const Frag* qf, float a, float b, float sc[4]) {
+// The 16 keys from `key0` on of key/value head `c` as A operands: lane l holds key l % 16, columns 32 s + 8 (l / 16) ..
+__device__ __forceinline__ void load_keys(const MixedGeometry& g, const Tile& t, const bf16_t* __restrict__ k_cache, int c, int key0,
+                                          Frag* kf) {
     const int lane = threadIdx.x & (KIPP_WAVE - 1), l16 = lane & 15, quarter = lane >> 4;
-    const int c = h / (g.n_q / g.n_kv);
-    const int key = min(key0 + l16, t.last);            // rows beyond the context are masked below; their loads stay inside it
+    const int key = min(key0 + l16, t.last);            // rows beyond the context are masked later; their loads stay inside it
     const bf16_t* row = k_cache + (((size_t)t.table[key / g.page] * g.n_kv + c) * g.page + key % g.page) * HEAD_DIM + 8 * quarter;
-    Frag kf[KSTEPS];
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) kf[s].u = *(const u32x4*)(row + 32 * s);
+}
+
+// S^T[key][row] of one head for the 16 keys from `key0` on: lane l gets keys key0 + 4 (l / 16) + v of row l % 16,
+// already scaled, biased by distance and masked (-inf).  `kf`: the keys as A operands, `qf`: the head's query rows
+// as B operands.
+__device__ __forceinline__ void scores16(const MixedGeometry& g, const Tile& t, int key0, const Frag* kf, const Frag* qf,
+                                         float a, float b, float sc[4]) {
+    const int lane = threadIdx.x & (KIPP_WAVE - 1), l16 = lane & 15, quarter = lane >> 4;
     f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[s].v, qf[s].v, acc, 0, 0, 0);
@@ -140,42 +149,71 @@ __global__ void __launch_bounds__(MX_THREADS) mixed_stats_kernel(MixedGeometry g
     const int item = blockIdx.x;
     const Tile t = tile_of(g, item);
     const int wave = threadIdx.x / KIPP_WAVE, lane = threadIdx.x & (KIPP_WAVE - 1);
+    const int group = g.n_q / g.n_kv, h0 = wave * HPW;
+    if (h0 >= g.n_q) return;
+    constexpr bool shared = SHARED_KV != 0;                 // the wave's heads read one key/value head
+    Frag qf[HPW][KSTEPS];
+    float a[HPW], b[HPW], m[HPW], l[HPW];
 #pragma unroll
     for (int hh = 0; hh < HPW; ++hh) {
-        const int h = wave * HPW + hh;
-        if (h >= g.n_q) break;
-        Frag qf[KSTEPS];
-        load_queries(t, q, g.n_q, h, qf);
-        const float a = g.r1 != nullptr ? g.r1[h] : 0.0f, b = g.r2 != nullptr ? g.r2[h] : 0.0f;
-        float m = -INFINITY, l = 0.0f;
-        for (int index = t.begin; index < t.end; ++index) {
-            const int key0 = key_tile(t, index) * MX_KEYS;
+        const int h = min(h0 + hh, g.n_q - 1);
+        load_queries(t, q, g.n_q, h, qf[hh]);
+        a[hh] = g.r1 != nullptr ? g.r1[h] : 0.0f;
+        b[hh] = g.r2 != nullptr ? g.r2[h] : 0.0f;
+        m[hh] = -INFINITY;
+        l[hh] = 0.0f;
+    }
+    Frag kf[MX_KEYS / 16][KSTEPS], next[MX_KEYS / 16][KSTEPS];
+    if (t.begin < t.end) {
+#pragma unroll
+        for (int kb = 0; kb < MX_KEYS / 16; ++kb) load_keys(g, t, k_cache, h0 / group, key_tile(t, t.begin) * MX_KEYS + 16 * kb, next[kb]);
+    }
+    for (int index = t.begin; index < t.end; ++index) {
+        const int key0 = key_tile(t, index) * MX_KEYS;
+#pragma unroll
+        for (int kb = 0; kb < MX_KEYS / 16; ++kb)
+#pragma unroll
+            for (int s = 0; s < KSTEPS; ++s) kf[kb][s] = next[kb][s];
+        if (index + 1 < t.end) {            // the next tile's keys are on their way while this one is scored
+#pragma unroll
+            for (int kb = 0; kb < MX_KEYS / 16; ++kb) load_keys(g, t, k_cache, h0 / group, key_tile(t, index + 1) * MX_KEYS + 16 * kb, next[kb]);
+        }
+#pragma unroll
+        for (int hh = 0; hh < HPW; ++hh) {
+            if (h0 + hh >= g.n_q) break;
 #pragma unroll
             for (int kb = 0; kb < MX_KEYS / 16; ++kb) {
+                Frag own[KSTEPS];
+                if (!shared && hh > 0) load_keys(g, t, k_cache, (h0 + hh) / group, key0 + 16 * kb, own);
                 float sc[4];
-                scores16(g, t, k_cache, h, key0 + 16 * kb, qf, a, b, sc);
-                const float m_new = fmaxf(m, fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])));
+                scores16(g, t, key0 + 16 * kb, (!shared && hh > 0) ? own : kf[kb], qf[hh], a[hh], b[hh], sc);
+                const float m_new = fmaxf(m[hh], fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])));
                 if (m_new != -INFINITY) {
                     float sum = 0.0f;
 #pragma unroll
                     for (int v = 0; v < 4; ++v) sum += __expf(sc[v] - m_new);       // exp(-inf) = 0
-                    l = l * __expf(m - m_new) + sum;
-                    m = m_new;
+                    l[hh] = l[hh] * __expf(m[hh] - m_new) + sum;
+                    m[hh] = m_new;
                 }
             }
         }
+    }
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh) {
+        if (h0 + hh >= g.n_q) break;
+        float mm = m[hh], ll = l[hh];
         // the four lanes that share a row
 #pragma unroll
         for (int off = 16; off <= 32; off <<= 1) {
-            const float m_o = __shfl_xor(m, off, KIPP_WAVE), l_o = __shfl_xor(l, off, KIPP_WAVE);
-            const float m_new = fmaxf(m, m_o);
-            if (m_new != -INFINITY) l = l * __expf(m - m_new) + l_o * __expf(m_o - m_new);
-            m = m_new;
+            const float m_o = __shfl_xor(mm, off, KIPP_WAVE), l_o = __shfl_xor(ll, off, KIPP_WAVE);
+            const float m_new = fmaxf(mm, m_o);
+            if (m_new != -INFINITY) ll = ll * __expf(mm - m_new) + l_o * __expf(m_o - m_new);
+            mm = m_new;
         }
         if (lane < 16) {
-            float* out = stats + (((size_t)item * g.n_q + h) * MX_ROWS + lane) * 2;
-            out[0] = m;
-            out[1] = l;
+            float* out = stats + (((size_t)item * g.n_q + h0 + hh) * MX_ROWS + lane) * 2;
+            out[0] = mm;
+            out[1] = ll;
         }
     }
 }
@@ -195,6 +233,7 @@ __global__ void __launch_bounds__(MX_THREADS) mixed_values_kernel(
     const int wave = threadIdx.x / KIPP_WAVE, lane = threadIdx.x & (KIPP_WAVE - 1), l16 = lane & 15, quarter = lane >> 4;
     const int nsplits = g.item_nsplits[item], split = g.item_split[item];
     const int n_q = g.n_q, group = g.n_q / g.n_kv;
+    constexpr bool shared = SHARED_KV != 0;                 // the wave's heads read one key/value head
 
     // columns of heads that do not exist stay zero for the whole walk
     for (int e = threadIdx.x; e < 2 * MX_ROWS * MX_KEYS * MX_HPAD / 8; e += MX_THREADS) ((u32x4*)p_hi)[e] = (u32x4){0u, 0u, 0u, 0u};
@@ -227,12 +266,18 @@ __global__ void __launch_bounds__(MX_THREADS) mixed_values_kernel(
             bias_a[hh] = g.r1 != nullptr ? g.r1[h] : 0.0f;
             bias_b[hh] = g.r2 != nullptr ? g.r2[h] : 0.0f;
             float m = sink != nullptr ? sink[h] : -INFINITY, l = sink != nullptr ? 1.0f : 0.0f;
-            for (int s = 0; s < nsplits; ++s) {
-                const float* st = stats + (((size_t)(item - split + s) * n_q + h) * MX_ROWS + l16) * 2;
-                const float m_s = st[0], l_s = st[1];
-                const float m_new = fmaxf(m, m_s);
-                if (m_new != -INFINITY) l = l * __expf(m - m_new) + l_s * __expf(m_s - m_new);
-                m = m_new;
+            for (int s0 = 0; s0 < nsplits; s0 += 4) {       // four runs' statistics asked for at once, then added in order
+                float2 st[4];
+#pragma unroll
+                for (int s = 0; s < 4; ++s)
+                    st[s] = s0 + s < nsplits ? *(const float2*)(stats + (((size_t)(item - split + s0 + s) * n_q + h) * MX_ROWS + l16) * 2)
+                                             : make_float2(-INFINITY, 0.0f);
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const float m_new = fmaxf(m, st[s].x);
+                    if (m_new != -INFINITY) l = l * __expf(m - m_new) + st[s].y * __expf(st[s].x - m_new);
+                    m = m_new;
+                }
             }
             top[hh] = m;
             inv[hh] = l > 0.0f ? 1.0f / l : 0.0f;
@@ -248,22 +293,27 @@ __global__ void __launch_bounds__(MX_THREADS) mixed_values_kernel(
 
     for (int index = t.begin; index < t.end; ++index) {
         const int key0 = key_tile(t, index) * MX_KEYS;
-        // 1. the final weights of this wave's heads
+        // 1. the final weights of this wave's heads; 16 keys are loaded once for all heads that share them
 #pragma unroll
-        for (int hh = 0; hh < HPW; ++hh) {
-            const int h = wave * HPW + hh;
-            if (h < n_q) {
+        for (int kb = 0; kb < MX_KEYS / 16; ++kb) {
+            if (wave * HPW < n_q) {
+                Frag kf[KSTEPS];
+                load_keys(g, t, k_cache, wave * HPW / group, key0 + 16 * kb, kf);
 #pragma unroll
-                for (int kb = 0; kb < MX_KEYS / 16; ++kb) {
-                    float sc[4];
-                    scores16(g, t, k_cache, h, key0 + 16 * kb, qf[hh], bias_a[hh], bias_b[hh], sc);
+                for (int hh = 0; hh < HPW; ++hh) {
+                    const int h = wave * HPW + hh;
+                    if (h < n_q) {
+                        if (!shared && hh > 0) load_keys(g, t, k_cache, h / group, key0 + 16 * kb, kf);
+                        float sc[4];
+                        scores16(g, t, key0 + 16 * kb, kf, qf[hh], bias_a[hh], bias_b[hh], sc);
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        const float p = sc[v] == -INFINITY ? 0.0f : __expf(sc[v] - top[hh]) * inv[hh];
-                        const bf16_t hi = f32_to_bf16(p);
-                        const int at = ((l16 * MX_KEYS) + 16 * kb + 4 * quarter + v) * MX_HPAD + h;
-                        p_hi[at] = hi;
-                        p_lo[at] = f32_to_bf16(p - bf16_to_f32(hi));
+                        for (int v = 0; v < 4; ++v) {
+                            const float p = sc[v] == -INFINITY ? 0.0f : __expf(sc[v] - top[hh]) * inv[hh];
+                            const bf16_t hi = f32_to_bf16(p);
+                            const int at = ((l16 * MX_KEYS) + 16 * kb + 4 * quarter + v) * MX_HPAD + h;
+                            p_hi[at] = hi;
+                            p_lo[at] = f32_to_bf16(p - bf16_to_f32(hi));
+                        }
                     }
                 }
             }
@@ -299,18 +349,41 @@ __global__ void __launch_bounds__(MX_THREADS) mixed_values_kernel(
         const int chunk = min(key0 + 8 * quarter, t.last);          // eight keys of one page (a page holds a multiple of 8)
         const size_t v_page = (size_t)t.table[chunk / g.page] * g.n_kv;
         const int v_slot = (key0 + 8 * quarter) % g.page;
+        if (shared) {
+            if (wave * HPW < n_q) {
+                const bf16_t* v_at = v_cache + ((v_page + wave * HPW / group) * V_DIM + l16) * g.page + v_slot;
+                constexpr int VB = VBLOCKS < 4 ? VBLOCKS : 4;        // value blocks asked for together
 #pragma unroll
-        for (int hh = 0; hh < HPW; ++hh) {
-            const int h = wave * HPW + hh;
-            if (h < n_q) {
-                Frag pf;
-                pf.u = *(const u32x4*)(p_mixed + ((size_t)(h * MX_ROWS + l16) * MX_KEYS + 8 * quarter));
-                const bf16_t* v_at = v_cache + ((v_page + h / group) * V_DIM + l16) * g.page + v_slot;
+                for (int m0 = 0; m0 < VBLOCKS; m0 += VB) {
+                    Frag vf[VB];
 #pragma unroll
-                for (int mb = 0; mb < VBLOCKS; ++mb) {
-                    Frag vf;
-                    vf.u = *(const u32x4*)(v_at + (size_t)16 * mb * g.page);
-                    acc[hh][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, acc[hh][mb], 0, 0, 0);
+                    for (int mb = 0; mb < VB; ++mb)
+                        if (m0 + mb < VBLOCKS) vf[mb].u = *(const u32x4*)(v_at + (size_t)16 * (m0 + mb) * g.page);
+#pragma unroll
+                    for (int hh = 0; hh < HPW; ++hh) {
+                        Frag pf;
+                        pf.u = *(const u32x4*)(p_mixed + ((size_t)(min(wave * HPW + hh, n_q - 1) * MX_ROWS + l16) * MX_KEYS + 8 * quarter));
+#pragma unroll
+                        for (int mb = 0; mb < VB; ++mb)
+                            if (m0 + mb < VBLOCKS && wave * HPW + hh < n_q)
+                                acc[hh][m0 + mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[mb].v, pf.v, acc[hh][m0 + mb], 0, 0, 0);
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int hh = 0; hh < HPW; ++hh) {
+                const int h = wave * HPW + hh;
+                if (h < n_q) {
+                    Frag pf;
+                    pf.u = *(const u32x4*)(p_mixed + ((size_t)(h * MX_ROWS + l16) * MX_KEYS + 8 * quarter));
+                    const bf16_t* v_at = v_cache + ((v_page + h / group) * V_DIM + l16) * g.page + v_slot;
+#pragma unroll
+                    for (int mb = 0; mb < VBLOCKS; ++mb) {
+                        Frag vf;
+                        vf.u = *(const u32x4*)(v_at + (size_t)16 * mb * g.page);
+                        acc[hh][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, acc[hh][mb], 0, 0, 0);
+                    }
                 }
             }
         }
@@ -350,24 +423,39 @@ __global__ void __launch_bounds__(MX_THREADS) mixed_values_kernel(
     }
 }
 
-// Rows whose keys were cut into runs: out = gate * (sum of the runs' partial sums, in order).
+// Rows whose keys were cut into runs: out = gate * (sum of the runs' partial sums, in order).  A thread takes four
+// columns of a row and asks for every run's sums before it adds the first.
 __global__ void __launch_bounds__(256) mixed_finish_kernel(const float* __restrict__ partial, size_t partial_stride,
                                                            const int32_t* __restrict__ row_splits, const float* __restrict__ gate,
                                                            int gate_stride, int gate_parts, size_t gate_part_stride,
                                                            bf16_t* __restrict__ out, int width) {
-    const size_t row = blockIdx.x;
+    const size_t row = blockIdx.y;
     const int n = row_splits[row];
-    if (n <= 1) return;
-    for (int e = threadIdx.x; e < width; e += 256) {
-        float o = 0.0f;
-        for (int s = 0; s < n; ++s) o += partial[s * partial_stride + row * width + e];
+    const int e = 4 * (blockIdx.x * 256 + threadIdx.x);
+    if (n <= 1 || e >= width) return;
+    f32x4 o = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int s0 = 0; s0 < n; s0 += 8) {
+        f32x4 part[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s)
+            part[s] = s0 + s < n ? *(const f32x4*)(partial + (s0 + s) * partial_stride + row * width + e) : (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int s = 0; s < 8; ++s) o += part[s];
+    }
+    float r[4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        r[v] = o[v];
         if (gate != nullptr) {
             float z = 0.0f;
-            for (int p = 0; p < gate_parts; ++p) z += gate[p * gate_part_stride + row * gate_stride + e];
-            o *= 1.0f / (1.0f + __expf(-z));
+            for (int p = 0; p < gate_parts; ++p) z += gate[p * gate_part_stride + row * gate_stride + e + v];
+            r[v] *= 1.0f / (1.0f + __expf(-z));
         }
-        out[row * width + e] = f32_to_bf16(o);
     }
+    uint2 w;
+    w.x = (uint32_t)f32_to_bf16(r[0]) | ((uint32_t)f32_to_bf16(r[1]) << 16);
+    w.y = (uint32_t)f32_to_bf16(r[2]) | ((uint32_t)f32_to_bf16(r[3]) << 16);
+    *(uint2*)(out + row * width + e) = w;
 }
 
 extern "C" {
@@ -394,6 +482,7 @@ int kipp_mixed_attention_mfma(const void* q, const void* k_cache, const void* v_
                               hipStream_t stream) {
     if (n_items <= 0 || n_rows <= 0) return 0;
     if (d != HEAD_DIM || dv != V_DIM || n_kv <= 0 || n_q % n_kv || n_q > MX_WAVES * HPW || n_q > MX_HPAD) return -1;
+    if (SHARED_KV && HPW > 1 && (n_q / n_kv) % HPW) return -4;
     if (page <= 0 || page % 16 || max_splits < 1 || (max_splits > 1 && (partial == nullptr || row_splits == nullptr))) return -2;
     MixedGeometry g;
     g.item_entry = item_entry; g.item_row0 = item_row0; g.item_split = item_split; g.item_nsplits = item_nsplits;
@@ -413,7 +502,7 @@ int kipp_mixed_attention_mfma(const void* q, const void* k_cache, const void* v_
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, stats, sink, mix, gate, gate_stride, gate_parts,
                        gate_part_stride, (bf16_t*)out, partial, partial_stride);
     if (max_splits > 1)
-        hipLaunchKernelGGL(mixed_finish_kernel, dim3(n_rows), dim3(256), 0, stream, partial, partial_stride, row_splits, gate,
+        hipLaunchKernelGGL(mixed_finish_kernel, dim3((n_q * V_DIM / 4 + 255) / 256, n_rows), dim3(256), 0, stream, partial, partial_stride, row_splits, gate,
                            gate_stride, gate_parts, gate_part_stride, (bf16_t*)out, n_q * V_DIM);
     return KIPP_LAUNCH_CHECK();
 }

@@ -324,6 +324,70 @@ __global__ void __launch_bounds__(256) scaled_add_rmsnorm_kernel(float* __restri
     }
 }
 
+// The same for widths that are a multiple of 4 and at most 1024 * CH: the row stays in registers, every load is asked
+// for before anything is added (slabs four at a time), 16-byte accesses.
+template <typename TD, typename TO, int CH>
+__global__ void __launch_bounds__(256) scaled_add_rmsnorm_rows_kernel(float* __restrict__ x, const TD* __restrict__ delta,
+                                                                      const float* __restrict__ weight, TO* __restrict__ rows,
+                                                                      int width, float eps, float alpha, int parts, size_t part_stride) {
+    __shared__ float scratch[16];
+    const int n4 = width / 4;
+    const size_t base4 = (size_t)blockIdx.x * n4;
+    float4 v[CH], w[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int i = threadIdx.x + c * 256;
+        v[c] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        w[c] = v[c];
+        if (i < n4) {
+            v[c] = load4(x, base4 + i);
+            w[c] = load4(weight, (size_t)i);
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        v[c].x *= alpha;
+        v[c].y *= alpha;
+        v[c].z *= alpha;
+        v[c].w *= alpha;
+    }
+    for (int p0 = 0; p0 < parts; p0 += 4) {
+        float4 d[CH][4];
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int i = threadIdx.x + c * 256;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                d[c][q] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                if (i < n4 && p0 + q < parts) d[c][q] = load4(delta, (p0 + q) * (part_stride / 4) + base4 + i);
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {   // slabs in order
+                v[c].x += d[c][q].x;
+                v[c].y += d[c][q].y;
+                v[c].z += d[c][q].z;
+                v[c].w += d[c][q].w;
+            }
+    }
+    float ss = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) ss += v[c].x * v[c].x + v[c].y * v[c].y + v[c].z * v[c].z + v[c].w * v[c].w;
+    ss = block_sum(ss, scratch);
+    const float scale = 1.0f / sqrtf(ss / (float)width + eps);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int i = threadIdx.x + c * 256;
+        if (i < n4) {
+            const float4 y = make_float4(v[c].x * scale * w[c].x, v[c].y * scale * w[c].y, v[c].z * scale * w[c].z, v[c].w * scale * w[c].w);
+            store4(x, base4 + i, y);
+            if (rows != nullptr) store4(rows, base4 + i, y);
+        }
+    }
+}
+
 template <typename TD, typename TO>
 static void launch_rmsnorm(float* x, const void* delta, const float* weight, void* out, int rows, int width, float eps,
                            int parts, hipStream_t stream) {
@@ -384,13 +448,26 @@ int kipp_scaled_add_rmsnorm(float* x, const void* delta, int delta_dtype, int pa
     if (n_rows <= 0 || width <= 0) return 0;
     if (parts < 0 || (parts > 0 && delta == nullptr)) return -1;
     const size_t stride = (size_t)n_rows * width;
-#define KIPP_PN(TD, TO) hipLaunchKernelGGL((scaled_add_rmsnorm_kernel<TD, TO>), dim3(n_rows), dim3(256), 0, stream, x, (const TD*)delta, weight, (TO*)rows, width, eps, alpha, parts, stride)
+    const int n4 = width / 4;
+    const bool in_registers = (width & 3) == 0 && n4 <= 256 * 8;
+#define KIPP_PR(TD, TO, CH) hipLaunchKernelGGL((scaled_add_rmsnorm_rows_kernel<TD, TO, CH>), dim3(n_rows), dim3(256), 0, stream, x, (const TD*)delta, weight, (TO*)rows, width, eps, alpha, parts, stride)
+#define KIPP_PN(TD, TO)                                                                                                           \
+    do {                                                                                                                          \
+        if (!in_registers)                                                                                                        \
+            hipLaunchKernelGGL((scaled_add_rmsnorm_kernel<TD, TO>), dim3(n_rows), dim3(256), 0, stream, x, (const TD*)delta, weight, \
+                               (TO*)rows, width, eps, alpha, parts, stride);                                                       \
+        else if (n4 <= 256) KIPP_PR(TD, TO, 1);                                                                                   \
+        else if (n4 <= 512) KIPP_PR(TD, TO, 2);                                                                                   \
+        else if (n4 <= 1024) KIPP_PR(TD, TO, 4);                                                                                  \
+        else KIPP_PR(TD, TO, 8);                                                                                                  \
+    } while (0)
     if (delta_dtype == KIPP_BF16) {
         if (rows_dtype == KIPP_BF16) KIPP_PN(bf16_t, bf16_t); else KIPP_PN(bf16_t, float);
     } else {
         if (rows_dtype == KIPP_BF16) KIPP_PN(float, bf16_t); else KIPP_PN(float, float);
     }
 #undef KIPP_PN
+#undef KIPP_PR
     return KIPP_LAUNCH_CHECK();
 }
 
