@@ -79,9 +79,10 @@ __global__ void __launch_bounds__(MIXED_THREADS) mixed_prepare_kernel(
 }
 
 // The same with a token's sums staged in LDS (dynamic, n_q d + n_kv d + n_kv dv floats): the slabs are read once, four
-// at a time, and every value is normed or written from LDS.  Same sums in the same order as the kernel above.
+// at a time, and every value is normed or written from LDS; few tokens get workgroups of 1,024 threads (the sums of
+// squares then add up in another order: the float32 path, whose bits must not depend on the batch, stays at 256).
 template <typename TQ, typename TC>
-__global__ void __launch_bounds__(MIXED_THREADS) mixed_prepare_lds_kernel(
+__global__ void __launch_bounds__(1024) mixed_prepare_lds_kernel(
     const float* __restrict__ proj, int parts, size_t part_stride, int stride, int k_at, int v_at,
     const float* __restrict__ q_weight, const float* __restrict__ k_weight, float eps,
     TQ* __restrict__ q_out, TC* __restrict__ k_cache, TC* __restrict__ v_cache,
@@ -94,7 +95,7 @@ __global__ void __launch_bounds__(MIXED_THREADS) mixed_prepare_lds_kernel(
     const int q_dim = n_q * d, k_dim = n_kv * d, v_dim = n_kv * dv;
     const int total = q_dim + k_dim + v_dim;
     float ss_q = 0.0f, ss_k = 0.0f;
-    for (int e = threadIdx.x; e < total; e += MIXED_THREADS) {
+    for (int e = threadIdx.x; e < total; e += blockDim.x) {
         const int col = e < q_dim ? e : (e < q_dim + k_dim ? k_at + e - q_dim : v_at + e - q_dim - k_dim);
         float v = 0.0f;
         for (int p0 = 0; p0 < parts; p0 += 4) {
@@ -115,7 +116,7 @@ __global__ void __launch_bounds__(MIXED_THREADS) mixed_prepare_lds_kernel(
     const int pos = positions[t];
     const int page_id = write_kv ? block_table[(size_t)seq_of_token[t] * max_blocks + pos / page] : 0;
     const int slot = pos % page;
-    for (int e = threadIdx.x; e < (write_kv ? total : q_dim); e += MIXED_THREADS) {
+    for (int e = threadIdx.x; e < (write_kv ? total : q_dim); e += blockDim.x) {
         const float v = sums[e];
         if (e < q_dim) {
             store_f(q_out, (size_t)t * q_dim + e, v * scale_q * q_weight[e]);
@@ -286,7 +287,7 @@ int kipp_mixed_prepare(const float* proj, int parts, int stride, int k_at, int v
 #define KIPP_MP(TQ, TC)                                                                                                    \
     do {                                                                                                                   \
         if (staged <= 48 * 1024)                                                                                           \
-            hipLaunchKernelGGL((mixed_prepare_lds_kernel<TQ, TC>), dim3(n_tokens), dim3(MIXED_THREADS), staged, stream, proj, \
+            hipLaunchKernelGGL((mixed_prepare_lds_kernel<TQ, TC>), dim3(n_tokens), dim3(sizeof(TQ) == 2 && n_tokens <= 256 ? 1024 : 256), staged, stream, proj, \
                                parts, part_stride, stride, k_at, v_at, q_weight, k_weight, eps, (TQ*)q_out, (TC*)k_cache,    \
                                (TC*)v_cache, positions, seq_of_token, block_table, max_blocks, n_q, n_kv, d, dv, page,      \
                                write_kv);                                                                                   \

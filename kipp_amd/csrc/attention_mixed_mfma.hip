@@ -236,7 +236,8 @@ __global__ void __launch_bounds__(MX_THREADS) mixed_values_kernel(
     constexpr bool shared = SHARED_KV != 0;                 // the wave's heads read one key/value head
 
     // columns of heads that do not exist stay zero for the whole walk
-    for (int e = threadIdx.x; e < 2 * MX_ROWS * MX_KEYS * MX_HPAD / 8; e += MX_THREADS) ((u32x4*)p_hi)[e] = (u32x4){0u, 0u, 0u, 0u};
+    if (n_q < MX_HPAD)
+        for (int e = threadIdx.x; e < 2 * MX_ROWS * MX_KEYS * MX_HPAD / 8; e += MX_THREADS) ((u32x4*)p_hi)[e] = (u32x4){0u, 0u, 0u, 0u};
 
     // mix^T as B operands: lane holds head (column) 16 nb + l % 16, contraction heads 8 (l / 16) ..
     Frag mf[2];
@@ -265,19 +266,33 @@ __global__ void __launch_bounds__(MX_THREADS) mixed_values_kernel(
             load_queries(t, q, n_q, h, qf[hh]);
             bias_a[hh] = g.r1 != nullptr ? g.r1[h] : 0.0f;
             bias_b[hh] = g.r2 != nullptr ? g.r2[h] : 0.0f;
-            float m = sink != nullptr ? sink[h] : -INFINITY, l = sink != nullptr ? 1.0f : 0.0f;
-            for (int s0 = 0; s0 < nsplits; s0 += 4) {       // four runs' statistics asked for at once, then added in order
+            // the runs' statistics: each quarter of the wave takes every fourth run (four asked for at once), the
+            // quarters are then merged, the sink last; any order gives the same maximum, and the sums differ in rounding only
+            float m = -INFINITY, l = 0.0f;
+            for (int s0 = quarter; s0 < nsplits; s0 += 16) {
                 float2 st[4];
 #pragma unroll
                 for (int s = 0; s < 4; ++s)
-                    st[s] = s0 + s < nsplits ? *(const float2*)(stats + (((size_t)(item - split + s0 + s) * n_q + h) * MX_ROWS + l16) * 2)
-                                             : make_float2(-INFINITY, 0.0f);
+                    st[s] = s0 + 4 * s < nsplits ? *(const float2*)(stats + (((size_t)(item - split + s0 + 4 * s) * n_q + h) * MX_ROWS + l16) * 2)
+                                                 : make_float2(-INFINITY, 0.0f);
 #pragma unroll
                 for (int s = 0; s < 4; ++s) {
                     const float m_new = fmaxf(m, st[s].x);
                     if (m_new != -INFINITY) l = l * __expf(m - m_new) + st[s].y * __expf(st[s].x - m_new);
                     m = m_new;
                 }
+            }
+#pragma unroll
+            for (int off = 16; off <= 32; off <<= 1) {
+                const float m_o = __shfl_xor(m, off, KIPP_WAVE), l_o = __shfl_xor(l, off, KIPP_WAVE);
+                const float m_new = fmaxf(m, m_o);
+                if (m_new != -INFINITY) l = l * __expf(m - m_new) + l_o * __expf(m_o - m_new);
+                m = m_new;
+            }
+            if (sink != nullptr) {
+                const float m_new = fmaxf(m, sink[h]);
+                l = (m == -INFINITY ? 0.0f : l * __expf(m - m_new)) + __expf(sink[h] - m_new);
+                m = m_new;
             }
             top[hh] = m;
             inv[hh] = l > 0.0f ? 1.0f / l : 0.0f;
