@@ -47,12 +47,30 @@
 #define MX_ROWS 16
 #define MX_KEYS 32
 #define MX_HPAD 32                      // heads padded to one step of the mixing product
+// LDS strides, in bfloat16 values, chosen so that the lanes of a wave fall into different banks: the weights as
+// [row][key][head] with 40 values a key (32 heads and 8 unused) and 1,288 a row, which a lane writes two bytes at a
+// time (16 rows x 4 keys of one head: 4 lanes a bank instead of 64 with the plain strides) and reads 16 bytes at a
+// time (no conflict); the mixed weights as [head][row][key] with 40 values a row and 656 a head.
+#define P_KEY 40
+#define P_ROW 1288
+#define M_ROW 40
+#define M_HEAD 656
+#define MX_LDS_BYTES ((2 * MX_ROWS * P_ROW + MX_HPAD * M_HEAD) * 2)
 #define KSTEPS (HEAD_DIM / 32)
-#define VBLOCKS (V_DIM / 16)
+#ifndef V_SLICE
+#define V_SLICE V_DIM                   // value columns a workgroup sums: V_DIM / V_SLICE workgroups share an item, each
+#endif                                  // with its own columns (their sums then fit a wave's registers) and all of the weights
+#define VBLOCKS (V_SLICE / 16)
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+// float32 -> bfloat16 by the hardware's conversion (round to nearest even, as f32_to_bf16 does for finite values)
+__device__ __forceinline__ bf16_t to_bf16(float f) {
+    const __bf16 b = (__bf16)f;
+    return __builtin_bit_cast(bf16_t, b);
+}
 
 union Frag {
     u32x4 u;
@@ -119,6 +137,7 @@ __device__ __forceinline__ void load_keys(const MixedGeometry& g, const Tile& t,
 // S^T[key][row] of one head for the 16 keys from `key0` on: lane l gets keys key0 + 4 (l / 16) + v of row l % 16,
 // already scaled, biased by distance and masked (-inf).  `kf`: the keys as A operands, `qf`: the head's query rows
 // as B operands.
+template <bool INSIDE>
 __device__ __forceinline__ void scores16(const MixedGeometry& g, const Tile& t, int key0, const Frag* kf, const Frag* qf,
                                          float a, float b, float sc[4]) {
     const int lane = threadIdx.x & (KIPP_WAVE - 1), l16 = lane & 15, quarter = lane >> 4;
@@ -129,9 +148,16 @@ __device__ __forceinline__ void scores16(const MixedGeometry& g, const Tile& t, 
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
         const int j = key0 + 4 * quarter + v;
-        const bool sees = l16 < t.rows && j <= i && (g.window <= 0 || i - j < g.window || j < g.keep_first);
+        // INSIDE: every row of the tile sees all 16 keys (rows that only fill the tile up compute unused numbers)
+        const bool sees = INSIDE || (l16 < t.rows && j <= i && (g.window <= 0 || i - j < g.window || j < g.keep_first));
         sc[v] = sees ? acc[v] * g.scale - a * __logf(1.0f + b * (float)(i - j)) : -INFINITY;
     }
+}
+
+// Whether every row of the tile sees every key of the 32 from `key0` on: behind the first row, and inside the window of
+// the last (or among the kept first keys).
+__device__ __forceinline__ bool all_seen(const MixedGeometry& g, const Tile& t, int key0) {
+    return key0 + MX_KEYS - 1 <= t.pos0 && (g.window <= 0 || t.pos0 + MX_ROWS - 1 - key0 < g.window || key0 + MX_KEYS <= g.keep_first);
 }
 
 // The query rows of head h as B operands: lane l holds row l % 16, columns 32 s + 8 (l / 16) ..
@@ -174,6 +200,7 @@ __global__ void __launch_bounds__(MX_THREADS) mixed_stats_kernel(MixedGeometry g
         for (int kb = 0; kb < MX_KEYS / 16; ++kb)
 #pragma unroll
             for (int s = 0; s < KSTEPS; ++s) kf[kb][s] = next[kb][s];
+        const bool inside = all_seen(g, t, key0);
         if (index + 1 < t.end) {            // the next tile's keys are on their way while this one is scored
 #pragma unroll
             for (int kb = 0; kb < MX_KEYS / 16; ++kb) load_keys(g, t, k_cache, h0 / group, key_tile(t, index + 1) * MX_KEYS + 16 * kb, next[kb]);
@@ -186,7 +213,8 @@ __global__ void __launch_bounds__(MX_THREADS) mixed_stats_kernel(MixedGeometry g
                 Frag own[KSTEPS];
                 if (!shared && hh > 0) load_keys(g, t, k_cache, (h0 + hh) / group, key0 + 16 * kb, own);
                 float sc[4];
-                scores16(g, t, key0 + 16 * kb, (!shared && hh > 0) ? own : kf[kb], qf[hh], a[hh], b[hh], sc);
+                if (inside) scores16<true>(g, t, key0 + 16 * kb, (!shared && hh > 0) ? own : kf[kb], qf[hh], a[hh], b[hh], sc);
+                else scores16<false>(g, t, key0 + 16 * kb, (!shared && hh > 0) ? own : kf[kb], qf[hh], a[hh], b[hh], sc);
                 const float m_new = fmaxf(m[hh], fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])));
                 if (m_new != -INFINITY) {
                     float sum = 0.0f;
@@ -218,7 +246,7 @@ __global__ void __launch_bounds__(MX_THREADS) mixed_stats_kernel(MixedGeometry g
     }
 }
 
-// LDS: p_hi, p_lo [16 rows][32 keys][32 heads] bfloat16, then p' [n_q][16 rows][32 keys] bfloat16.
+// LDS: p_hi, p_lo [16 rows][32 keys][32 heads] bfloat16, then p' [32 heads][16 rows][32 keys] bfloat16, with the padded strides above.
 __global__ void __launch_bounds__(MX_THREADS) mixed_values_kernel(
     MixedGeometry g, const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const float* __restrict__ stats, const float* __restrict__ sink, const float* __restrict__ mix,
@@ -226,9 +254,9 @@ __global__ void __launch_bounds__(MX_THREADS) mixed_values_kernel(
     bf16_t* __restrict__ out, float* __restrict__ partial, size_t partial_stride) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     bf16_t* p_hi = (bf16_t*)lds_raw;
-    bf16_t* p_lo = p_hi + MX_ROWS * MX_KEYS * MX_HPAD;
-    bf16_t* p_mixed = p_lo + MX_ROWS * MX_KEYS * MX_HPAD;
-    const int item = blockIdx.x;
+    bf16_t* p_lo = p_hi + MX_ROWS * P_ROW;
+    bf16_t* p_mixed = p_lo + MX_ROWS * P_ROW;
+    const int item = blockIdx.x, v0 = blockIdx.y * V_SLICE;        // this workgroup's value columns v0 .. v0 + V_SLICE - 1 of every head
     const Tile t = tile_of(g, item);
     const int wave = threadIdx.x / KIPP_WAVE, lane = threadIdx.x & (KIPP_WAVE - 1), l16 = lane & 15, quarter = lane >> 4;
     const int nsplits = g.item_nsplits[item], split = g.item_split[item];
@@ -237,7 +265,7 @@ __global__ void __launch_bounds__(MX_THREADS) mixed_values_kernel(
 
     // columns of heads that do not exist stay zero for the whole walk
     if (n_q < MX_HPAD)
-        for (int e = threadIdx.x; e < 2 * MX_ROWS * MX_KEYS * MX_HPAD / 8; e += MX_THREADS) ((u32x4*)p_hi)[e] = (u32x4){0u, 0u, 0u, 0u};
+        for (int e = threadIdx.x; e < 2 * MX_ROWS * P_ROW / 8; e += MX_THREADS) ((u32x4*)p_hi)[e] = (u32x4){0u, 0u, 0u, 0u};
 
     // mix^T as B operands: lane holds head (column) 16 nb + l % 16, contraction heads 8 (l / 16) ..
     Frag mf[2];
@@ -308,26 +336,49 @@ __global__ void __launch_bounds__(MX_THREADS) mixed_values_kernel(
 
     for (int index = t.begin; index < t.end; ++index) {
         const int key0 = key_tile(t, index) * MX_KEYS;
-        // 1. the final weights of this wave's heads; 16 keys are loaded once for all heads that share them
+        const bool inside = all_seen(g, t, key0);
+        // 1. the final weights of this wave's heads; 16 keys are loaded once for all heads that share them, and a lane
+        //    writes the weights of its heads (they are neighbours in the [row][key][head] layout) with one store
 #pragma unroll
         for (int kb = 0; kb < MX_KEYS / 16; ++kb) {
             if (wave * HPW < n_q) {
                 Frag kf[KSTEPS];
                 load_keys(g, t, k_cache, wave * HPW / group, key0 + 16 * kb, kf);
+                float p[HPW][4];
 #pragma unroll
                 for (int hh = 0; hh < HPW; ++hh) {
                     const int h = wave * HPW + hh;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) p[hh][v] = 0.0f;
                     if (h < n_q) {
                         if (!shared && hh > 0) load_keys(g, t, k_cache, h / group, key0 + 16 * kb, kf);
                         float sc[4];
-                        scores16(g, t, key0 + 16 * kb, kf, qf[hh], bias_a[hh], bias_b[hh], sc);
+                        if (inside) scores16<true>(g, t, key0 + 16 * kb, kf, qf[hh], bias_a[hh], bias_b[hh], sc);
+                        else scores16<false>(g, t, key0 + 16 * kb, kf, qf[hh], bias_a[hh], bias_b[hh], sc);
 #pragma unroll
-                        for (int v = 0; v < 4; ++v) {
-                            const float p = sc[v] == -INFINITY ? 0.0f : __expf(sc[v] - top[hh]) * inv[hh];
-                            const bf16_t hi = f32_to_bf16(p);
-                            const int at = ((l16 * MX_KEYS) + 16 * kb + 4 * quarter + v) * MX_HPAD + h;
-                            p_hi[at] = hi;
-                            p_lo[at] = f32_to_bf16(p - bf16_to_f32(hi));
+                        for (int v = 0; v < 4; ++v) p[hh][v] = sc[v] == -INFINITY ? 0.0f : __expf(sc[v] - top[hh]) * inv[hh];
+                    }
+                }
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int at = l16 * P_ROW + (16 * kb + 4 * quarter + v) * P_KEY + wave * HPW;
+                    bf16_t hi[HPW], lo[HPW];
+#pragma unroll
+                    for (int hh = 0; hh < HPW; ++hh) {
+                        hi[hh] = to_bf16(p[hh][v]);
+                        lo[hh] = to_bf16(p[hh][v] - bf16_to_f32(hi[hh]));
+                    }
+                    if (HPW == 4) {
+                        *(uint2*)(p_hi + at) = make_uint2((uint32_t)hi[0] | ((uint32_t)hi[1 % HPW] << 16), (uint32_t)hi[2 % HPW] | ((uint32_t)hi[3 % HPW] << 16));
+                        *(uint2*)(p_lo + at) = make_uint2((uint32_t)lo[0] | ((uint32_t)lo[1 % HPW] << 16), (uint32_t)lo[2 % HPW] | ((uint32_t)lo[3 % HPW] << 16));
+                    } else if (HPW == 2) {
+                        *(uint32_t*)(p_hi + at) = (uint32_t)hi[0] | ((uint32_t)hi[1 % HPW] << 16);
+                        *(uint32_t*)(p_lo + at) = (uint32_t)lo[0] | ((uint32_t)lo[1 % HPW] << 16);
+                    } else {
+#pragma unroll
+                        for (int hh = 0; hh < HPW; ++hh) {
+                            p_hi[at + hh] = hi[hh];
+                            p_lo[at + hh] = lo[hh];
                         }
                     }
                 }
@@ -339,7 +390,7 @@ __global__ void __launch_bounds__(MX_THREADS) mixed_values_kernel(
         for (int u = 0; u < (MX_ROWS * MX_KEYS / 16) / MX_WAVES; ++u) {
             const int block = wave + MX_WAVES * u;              // row = block / 2, keys 16 (block % 2) ..
             const int row = block >> 1, kb = block & 1;
-            const int at = ((row * MX_KEYS) + 16 * kb + l16) * MX_HPAD + 8 * quarter;
+            const int at = row * P_ROW + (16 * kb + l16) * P_KEY + 8 * quarter;
             Frag hi, lo;
             hi.u = *(const u32x4*)(p_hi + at);
             lo.u = *(const u32x4*)(p_lo + at);
@@ -352,9 +403,9 @@ __global__ void __launch_bounds__(MX_THREADS) mixed_values_kernel(
                     const int h = 16 * nb + l16;        // d[v]: keys 16 kb + 4 quarter + v of `row`, head h
                     if (h < n_q) {
                         uint2 w;
-                        w.x = (uint32_t)f32_to_bf16(d[0]) | ((uint32_t)f32_to_bf16(d[1]) << 16);
-                        w.y = (uint32_t)f32_to_bf16(d[2]) | ((uint32_t)f32_to_bf16(d[3]) << 16);
-                        *(uint2*)(p_mixed + ((size_t)(h * MX_ROWS + row) * MX_KEYS + 16 * kb + 4 * quarter)) = w;
+                        w.x = (uint32_t)to_bf16(d[0]) | ((uint32_t)to_bf16(d[1]) << 16);
+                        w.y = (uint32_t)to_bf16(d[2]) | ((uint32_t)to_bf16(d[3]) << 16);
+                        *(uint2*)(p_mixed + (h * M_HEAD + row * M_ROW + 16 * kb + 4 * quarter)) = w;
                     }
                 }
             }
@@ -366,7 +417,7 @@ __global__ void __launch_bounds__(MX_THREADS) mixed_values_kernel(
         const int v_slot = (key0 + 8 * quarter) % g.page;
         if (shared) {
             if (wave * HPW < n_q) {
-                const bf16_t* v_at = v_cache + ((v_page + wave * HPW / group) * V_DIM + l16) * g.page + v_slot;
+                const bf16_t* v_at = v_cache + ((v_page + wave * HPW / group) * V_DIM + v0 + l16) * g.page + v_slot;
                 constexpr int VB = VBLOCKS < 4 ? VBLOCKS : 4;        // value blocks asked for together
 #pragma unroll
                 for (int m0 = 0; m0 < VBLOCKS; m0 += VB) {
@@ -377,7 +428,7 @@ __global__ void __launch_bounds__(MX_THREADS) mixed_values_kernel(
 #pragma unroll
                     for (int hh = 0; hh < HPW; ++hh) {
                         Frag pf;
-                        pf.u = *(const u32x4*)(p_mixed + ((size_t)(min(wave * HPW + hh, n_q - 1) * MX_ROWS + l16) * MX_KEYS + 8 * quarter));
+                        pf.u = *(const u32x4*)(p_mixed + (min(wave * HPW + hh, n_q - 1) * M_HEAD + l16 * M_ROW + 8 * quarter));
 #pragma unroll
                         for (int mb = 0; mb < VB; ++mb)
                             if (m0 + mb < VBLOCKS && wave * HPW + hh < n_q)
@@ -391,8 +442,8 @@ __global__ void __launch_bounds__(MX_THREADS) mixed_values_kernel(
                 const int h = wave * HPW + hh;
                 if (h < n_q) {
                     Frag pf;
-                    pf.u = *(const u32x4*)(p_mixed + ((size_t)(h * MX_ROWS + l16) * MX_KEYS + 8 * quarter));
-                    const bf16_t* v_at = v_cache + ((v_page + h / group) * V_DIM + l16) * g.page + v_slot;
+                    pf.u = *(const u32x4*)(p_mixed + (h * M_HEAD + l16 * M_ROW + 8 * quarter));
+                    const bf16_t* v_at = v_cache + ((v_page + h / group) * V_DIM + v0 + l16) * g.page + v_slot;
 #pragma unroll
                     for (int mb = 0; mb < VBLOCKS; ++mb) {
                         Frag vf;
@@ -415,7 +466,7 @@ __global__ void __launch_bounds__(MX_THREADS) mixed_values_kernel(
         if (h >= n_q) break;
 #pragma unroll
         for (int mb = 0; mb < VBLOCKS; ++mb) {
-            const int col = h * V_DIM + 16 * mb + 4 * quarter;
+            const int col = h * V_DIM + v0 + 16 * mb + 4 * quarter;
             if (nsplits > 1) {
                 *(f32x4*)(partial + split * partial_stride + row * ((size_t)n_q * V_DIM) + col) = acc[hh][mb];
             } else {
@@ -479,7 +530,7 @@ int kipp_mixed_mfma_sizes(int* head_dim, int* v_dim, int* heads_per_wave, int* l
     *head_dim = HEAD_DIM;
     *v_dim = V_DIM;
     *heads_per_wave = HPW;
-    *lds_bytes = (2 * MX_ROWS * MX_KEYS * MX_HPAD + MX_HPAD * MX_ROWS * MX_KEYS) * 2;
+    *lds_bytes = MX_LDS_BYTES;
     return 0;
 }
 
@@ -496,6 +547,7 @@ int kipp_mixed_attention_mfma(const void* q, const void* k_cache, const void* v_
                               int n_rows, int n_q, int n_kv, int d, int dv, int page, float scale, int window, int keep_first,
                               hipStream_t stream) {
     if (n_items <= 0 || n_rows <= 0) return 0;
+    if (V_DIM % V_SLICE || V_SLICE % 16) return -5;
     if (d != HEAD_DIM || dv != V_DIM || n_kv <= 0 || n_q % n_kv || n_q > MX_WAVES * HPW || n_q > MX_HPAD) return -1;
     if (SHARED_KV && HPW > 1 && (n_q / n_kv) % HPW) return -4;
     if (page <= 0 || page % 16 || max_splits < 1 || (max_splits > 1 && (partial == nullptr || row_splits == nullptr))) return -2;
@@ -504,7 +556,7 @@ int kipp_mixed_attention_mfma(const void* q, const void* k_cache, const void* v_
     g.q_start = q_start; g.q_len = q_len; g.ctx_len = ctx_len; g.block_table = block_table;
     g.max_blocks = max_blocks; g.page = page; g.n_q = n_q; g.n_kv = n_kv; g.window = window; g.keep_first = keep_first;
     g.scale = scale; g.r1 = r1; g.r2 = r2;
-    const int lds = (2 * MX_ROWS * MX_KEYS * MX_HPAD + MX_HPAD * MX_ROWS * MX_KEYS) * 2;
+    const int lds = MX_LDS_BYTES;
     static bool raised = false;
     if (!raised) {
         if (hipFuncSetAttribute((const void*)mixed_values_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return -3;
@@ -513,7 +565,7 @@ int kipp_mixed_attention_mfma(const void* q, const void* k_cache, const void* v_
     const size_t gate_part_stride = (size_t)n_rows * gate_stride;
     const size_t partial_stride = (size_t)n_rows * n_q * V_DIM;
     hipLaunchKernelGGL(mixed_stats_kernel, dim3(n_items), dim3(MX_THREADS), 0, stream, g, (const bf16_t*)q, (const bf16_t*)k_cache, stats);
-    hipLaunchKernelGGL(mixed_values_kernel, dim3(n_items), dim3(MX_THREADS), lds, stream, g, (const bf16_t*)q,
+    hipLaunchKernelGGL(mixed_values_kernel, dim3(n_items, V_DIM / V_SLICE), dim3(MX_THREADS), lds, stream, g, (const bf16_t*)q,
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, stats, sink, mix, gate, gate_stride, gate_parts,
                        gate_part_stride, (bf16_t*)out, partial, partial_stride);
     if (max_splits > 1)

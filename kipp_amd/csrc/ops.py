@@ -394,10 +394,21 @@ MIXED_KEYS = 32         # keys it takes at a time
 MIXED_WAVES = 8
 
 
-def mixed_attention_defines(n_q: int, n_kv: int, d: int, dv: int) -> dict:
-    """The build of attention_mixed_mfma.hip that takes these sizes."""
+def mixed_attention_defines(n_q: int, n_kv: int, d: int, dv: int, sliced: bool = False) -> dict:
+    """The build of attention_mixed_mfma.hip that takes these sizes.  `sliced`: the build in which several workgroups
+    share an item, each with a part of the value columns (and all of the weights, computed again): twice the workgroups
+    for a step that leaves compute units idle, and a wave's sums within 64 registers."""
     hpw = -(-n_q // MIXED_WAVES)
-    return {"HEAD_DIM": d, "V_DIM": dv, "HPW": hpw, "SHARED_KV": int(hpw == 1 or (n_q // n_kv) % hpw == 0)}
+    blocks = dv // 16
+    while sliced and hpw * blocks > 16 and blocks % 2 == 0:
+        blocks //= 2
+    return {"HEAD_DIM": d, "V_DIM": dv, "HPW": hpw, "SHARED_KV": int(hpw == 1 or (n_q // n_kv) % hpw == 0), "V_SLICE": 16 * blocks}
+
+
+def mixed_attention_builds(n_q: int, n_kv: int, d: int, dv: int) -> list:
+    """Both builds (one where slicing changes nothing)."""
+    whole, sliced = mixed_attention_defines(n_q, n_kv, d, dv), mixed_attention_defines(n_q, n_kv, d, dv, sliced=True)
+    return [whole] if whole == sliced else [whole, sliced]
 
 
 def mixed_attention_fast_ok(n_q: int, d: int, dv: int, page: int) -> bool:
@@ -445,7 +456,9 @@ def mixed_attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.
           "mixed_attention_mfma: one q_start, q_len, ctx_len and table row an entry")
     fn = _fn("attention_mixed_mfma", "kipp_mixed_attention_mfma",
              [_c_ptr] * 5 + [_c_int, _c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr, _c_int] + [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 6
-             + [_c_int] * 6 + [_c_float, _c_int, _c_int, _c_ptr], mixed_attention_defines(n_q, n_kv, d, dv))
+             + [_c_int] * 6 + [_c_float, _c_int, _c_int, _c_ptr],
+             # fewer items than compute units: the value columns are shared out over more workgroups
+             mixed_attention_defines(n_q, n_kv, d, dv, sliced=n_items < COMPUTE_UNITS))
     gate_ptr = gate.data_ptr() + 4 * gate_at if gate is not None else None
     _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), gate_ptr, gate_stride, gate_parts,
               _ptr(items[0]), _ptr(items[1]), _ptr(items[2]), _ptr(items[3]), n_items, _ptr(row_splits), max_splits,

@@ -77,9 +77,9 @@ def check_builds() -> List[Spec]:
         out.append(("attention_decode", {"HEAD_DIM": head_dim, "GROUP": group, "STREAM_FROM": 1024}))
     for head_dim, group in WHOLE_CONTEXTS:
         out.append(("attention_decode", {"HEAD_DIM": head_dim, "GROUP": group, "RING_FROM_PAIRS": 1}))
-    from .ops import mixed_attention_defines
+    from .ops import mixed_attention_builds
     for heads, kv_heads, head_dim, v_dim in MIXED_HEADS:
-        out.append(("attention_mixed_mfma", mixed_attention_defines(heads, kv_heads, head_dim, v_dim)))
+        out += [("attention_mixed_mfma", defines) for defines in mixed_attention_builds(heads, kv_heads, head_dim, v_dim)]
     seen, unique = set(), []
     for name, defines in out:
         key = (name, tuple(sorted(defines.items())))

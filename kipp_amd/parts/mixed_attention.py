@@ -68,7 +68,8 @@ class MixedHeadAttention:
         from ..csrc import ops
         out = [("attention_mixed", None)]
         if dtype == "bfloat16" and ops.mixed_attention_fast_ok(spec.num_heads, spec.head_dim, spec.v_head_dim, spec.page_size or 16):
-            out.append(("attention_mixed_mfma", ops.mixed_attention_defines(spec.num_heads, spec.num_kv_heads, spec.head_dim, spec.v_head_dim)))
+            out += [("attention_mixed_mfma", defines)
+                    for defines in ops.mixed_attention_builds(spec.num_heads, spec.num_kv_heads, spec.head_dim, spec.v_head_dim)]
         return out
 
     def load(self, tensors):
