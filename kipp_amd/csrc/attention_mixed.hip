@@ -81,6 +81,7 @@ __global__ void __launch_bounds__(MIXED_THREADS) mixed_prepare_kernel(
 // The same with a token's sums staged in LDS (dynamic, n_q d + n_kv d + n_kv dv floats): the slabs are read once, four
 // at a time, and every value is normed or written from LDS; few tokens get workgroups of 1,024 threads (the sums of
 // squares then add up in another order: the float32 path, whose bits must not depend on the batch, stays at 256).
+// The order of a token's additions follows from the sizes alone.
 template <typename TQ, typename TC>
 __global__ void __launch_bounds__(1024) mixed_prepare_lds_kernel(
     const float* __restrict__ proj, int parts, size_t part_stride, int stride, int k_at, int v_at,
@@ -88,26 +89,51 @@ __global__ void __launch_bounds__(1024) mixed_prepare_lds_kernel(
     TQ* __restrict__ q_out, TC* __restrict__ k_cache, TC* __restrict__ v_cache,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
     const int32_t* __restrict__ block_table, int max_blocks, int n_q, int n_kv, int d, int dv, int page, int write_kv) {
-    extern __shared__ float sums[];
+    extern __shared__ __attribute__((aligned(16))) float sums[];
     __shared__ float scratch[16];
     const int t = blockIdx.x;
     const float* row = proj + (size_t)t * stride;
     const int q_dim = n_q * d, k_dim = n_kv * d, v_dim = n_kv * dv;
     const int total = q_dim + k_dim + v_dim;
     float ss_q = 0.0f, ss_k = 0.0f;
-    for (int e = threadIdx.x; e < total; e += blockDim.x) {
-        const int col = e < q_dim ? e : (e < q_dim + k_dim ? k_at + e - q_dim : v_at + e - q_dim - k_dim);
-        float v = 0.0f;
-        for (int p0 = 0; p0 < parts; p0 += 4) {
-            float part[4];
+    if (((q_dim | k_dim | v_dim | k_at | v_at | stride) & 3) == 0) {
+        // four columns a lane and load (every run of columns begins at a multiple of four, so a group never straddles two)
+        for (int e = 4 * threadIdx.x; e < total; e += 4 * blockDim.x) {
+            const int col = e < q_dim ? e : (e < q_dim + k_dim ? k_at + e - q_dim : v_at + e - q_dim - k_dim);
+            float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            for (int p0 = 0; p0 < parts; p0 += 4) {
+                float4 part[4];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) part[u] = p0 + u < parts ? row[(p0 + u) * part_stride + col] : 0.0f;
+                for (int u = 0; u < 4; ++u)
+                    part[u] = p0 + u < parts ? *(const float4*)(row + (p0 + u) * part_stride + col) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 #pragma unroll
-            for (int u = 0; u < 4; ++u) v += part[u];
+                for (int u = 0; u < 4; ++u) {
+                    v.x += part[u].x;
+                    v.y += part[u].y;
+                    v.z += part[u].z;
+                    v.w += part[u].w;
+                }
+            }
+            *(float4*)(sums + e) = v;
+            const float sq = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, v.w * v.w)));
+            if (e < q_dim) ss_q += sq;
+            else if (e < q_dim + k_dim) ss_k += sq;
         }
-        sums[e] = v;
-        if (e < q_dim) ss_q = fmaf(v, v, ss_q);
-        else if (e < q_dim + k_dim) ss_k = fmaf(v, v, ss_k);
+    } else {
+        for (int e = threadIdx.x; e < total; e += blockDim.x) {
+            const int col = e < q_dim ? e : (e < q_dim + k_dim ? k_at + e - q_dim : v_at + e - q_dim - k_dim);
+            float v = 0.0f;
+            for (int p0 = 0; p0 < parts; p0 += 4) {
+                float part[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) part[u] = p0 + u < parts ? row[(p0 + u) * part_stride + col] : 0.0f;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) v += part[u];
+            }
+            sums[e] = v;
+            if (e < q_dim) ss_q = fmaf(v, v, ss_q);
+            else if (e < q_dim + k_dim) ss_k = fmaf(v, v, ss_k);
+        }
     }
     ss_q = block_sum(ss_q, scratch);
     ss_k = block_sum(ss_k, scratch);
