@@ -17,7 +17,8 @@ from typing import List, Optional, Tuple
 Spec = Tuple[str, Optional[dict]]
 
 GENERIC: List[Spec] = [(name, None) for name in
-                       ("elementwise", "rope_kv", "attention_generic", "gemm_f32", "gemm_skinny", "gemm_rows", "gemm_tiles", "sampling")]
+                       ("elementwise", "gemm_f32", "gemm_skinny", "gemm_rows", "gemm_tiles", "sampling")]
+BF16_ONLY = ("gemm_skinny", "gemm_rows", "gemm_tiles")      # the matrix-core products: the float32 path never launches them
 
 
 def _add(out: List[Spec], more) -> None:
@@ -29,7 +30,7 @@ def _add(out: List[Spec], more) -> None:
 def model_variants(spec, dtype: str) -> List[Spec]:
     """Everything the model `spec` launches under `dtype`: the common files and what its parts declare."""
     from ..parts import part_class
-    out = list(GENERIC)
+    out = [v for v in GENERIC if dtype != "float32" or v[0] not in BF16_ONLY]
     owners = [("embedding", spec.embedding), ("norm", spec.final_norm), ("head", spec.head)]
     if getattr(spec, "input_position", None) is not None:
         owners.append(("position", spec.input_position))
@@ -48,7 +49,7 @@ def prebuilt() -> List[Spec]:
     """What `build()` compiles ahead: everything the named shapes under `config/shapes` launch, in both
     precisions, and the read-bandwidth yardstick of `python -m kipp_amd.workloads hbm`."""
     from ..config import parse_config, shape_config, shape_names
-    out = list(GENERIC)
+    out = list(GENERIC) + [("rope_kv", None), ("attention_generic", None)]
     for name in shape_names():
         _, cfg = parse_config(shape_config(name))
         for dtype in ("bfloat16", "float32"):

@@ -63,10 +63,11 @@ class Attention:
         """The builds of its specialised kernels (one per head size; decode also per number of query heads
         that share a key/value head).  Under float32, and for more than 16 heads a group, the generic
         attention kernel runs, which every model has."""
+        out = [("rope_kv", None), ("attention_generic", None)]
         if dtype != "bfloat16" or spec.head_dim % 16:
-            return []
+            return out
         group = spec.num_heads // spec.num_kv_heads
-        out = [("attention_prefill", {"HEAD_DIM": spec.head_dim})]
+        out.append(("attention_prefill", {"HEAD_DIM": spec.head_dim}))
         if group <= 16:
             out.append(("attention_decode", {"HEAD_DIM": spec.head_dim, "GROUP": group}))
         return out
