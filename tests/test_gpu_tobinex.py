@@ -270,6 +270,26 @@ def test_cuttings_match_plain(folders, shape, dtype, page, cut):
     assert (engine.rt.generic_attention_launches > 0) == (dtype == "bfloat16" and (page == 8 or shape == "tobinex-tiny-b"))
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("width, ff, heads", [(100, 52, (3, 1, 20, 12)), (72, 200, (2, 2, 36, 28)), (160, 88, (16, 4, 32, 16))])
+def test_sizes_that_leave_the_fast_kernels(tmp_path, dtype, width, ff, heads):
+    """Widths that are no multiple of 8 or of 32 (their products go to other kernels or to the library's), head sizes
+    only the plain attention takes, prompts longer than the few-rows and staged-rows products take, a vocabulary that is
+    no multiple of anything."""
+    from kipp_amd.weights import write_random_model
+    H_, G, d, dv = heads
+    cfg = {"architecture": "Tobinex", "vocab": 77, "width": width, "embedding": {"scale": 3.0}, "norm": {"eps": 1e-5}, "postln_alpha": 0.8,
+           "layers": [{"type": "attention", "mlp": {"kind": "dense", "ff": ff},
+                       "mixer": {"heads": H_, "kv_heads": G, "dim": d, "vdim": dv, "scale": 0.3, "mask": {"size": 50 + 7 * i, "keep_first": 2 * i}}}
+                      for i in range(2)]}
+    folder = write_random_model(str(tmp_path / "odd"), cfg, seed=width, dtype=dtype)
+    requests = {"long": H.random_tokens(1, 330, 77), "short": H.random_tokens(2, 9, 77)}
+    for steps in (H.whole(requests), [([("long", 270)], []), ([("long", 59), ("short", 8)], []), ([("long", 1), ("short", 1)], ["long", "short"])]):
+        got = H.replay(engine_of(folder, dtype), requests, steps)
+        for rid, toks in requests.items():
+            close(got[rid], plain_logits(folder, toks), TOL[dtype], f"{width}/{dtype}/{rid}")
+
+
 @pytest.mark.parametrize("shape", SHAPES)
 def test_float32_cuttings_are_bitwise_equal(folders, shape):
     """In float32 every sum runs in an order that the token's own position fixes: how the prompt was cut, what else was
