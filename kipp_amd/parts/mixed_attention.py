@@ -112,7 +112,7 @@ class MixedHeadAttention:
         gate_at = s.q_dim + s.kv_dim + s.v_dim
         if rt.dtype == "bfloat16" and getattr(rt, "mixed_attention_fast", True) \
                 and ops.mixed_attention_fast_ok(s.num_heads, s.head_dim, s.v_head_dim, cache.page_size):
-            items, n_items, row_splits, max_splits, workspace = self._work(batch)
+            items, n_items, row_splits, max_splits, workspace = self._items(batch)
             ops.mixed_attention_mfma(q, cache.k, cache.v, out, items, n_items, row_splits, max_splits,
                                      batch.q_start, batch.q_len, batch.ctx_len, table,
                                      s.num_heads, s.num_kv_heads, s.head_dim, s.v_head_dim, s.scale, s.window or 0,
@@ -127,7 +127,7 @@ class MixedHeadAttention:
                                   gate=proj if s.output_gate else None, gate_at=gate_at)
         return rt.linear(out, self.w_o, slabs=True, defer=True)
 
-    def _work(self, batch):
+    def _items(self, batch):
         """The item list of the matrix-core form: every entry's rows in tiles of 16, and where the tiles alone are too
         few workgroups to fill the GPU, each tile's keys in several runs (at least 128 keys a run, at most 16 runs).
         Made by the first layer of a geometry and kept while the batch object lives: a recorded step keeps its own,
