@@ -13,8 +13,9 @@ from dataclasses import dataclass
 from typing import Callable, Dict
 
 from .specs import (AttentionSpec, ConfigError, EmbeddingSpec, GatedMLPSpec,
-                    HeadSpec, LayerRun, LayerSpec, MixedHeadAttentionSpec, ModelSpec,
-                    NoPositionSpec, OnePlusRMSNormSpec, RMSNormSpec, RopeSpec)
+                    HeadSpec, HyperConnectionSpec, LatentAttentionSpec, LayerRun, LayerSpec, MLSTMSpec,
+                    MixedHeadAttentionSpec, ModelSpec, NoPositionSpec, OnePlusRMSNormSpec, RMSNormSpec, RopeSpec,
+                    ScaledRopeSpec)
 
 
 @dataclass(frozen=True)
@@ -98,3 +99,8 @@ from . import tobinex as _tobinex  # noqa: E402
 
 register_architecture(_tobinex.ARCHITECTURE, _tobinex.TobinexConfig.from_dict)
 TobinexConfig = _tobinex.TobinexConfig
+
+from . import rerizen as _rerizen  # noqa: E402
+
+register_architecture(_rerizen.ARCHITECTURE, _rerizen.RerizenConfig.from_dict)
+RerizenConfig = _rerizen.RerizenConfig

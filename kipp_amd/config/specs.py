@@ -27,6 +27,7 @@ class RMSNormSpec:
     eps: float
     prefix: str = ""
     kind: str = "rms_norm"
+    name: str = "weight"        # the tensor's local name (file name = prefix + name)
 
 
 @dataclass(frozen=True)
@@ -64,6 +65,36 @@ class RopeSpec:
 
 
 @dataclass(frozen=True)
+class ScaledRopeSpec:
+    """Rotary position encoding whose frequencies are stretched for contexts beyond the `original` length (the
+    YaRN rule).  With f_i = theta^(-2i / rotary_dim), i < rotary_dim / 2, and
+    turn(t) = rotary_dim * ln(original / (2 pi t)) / (2 ln theta), the dimension that makes t turns over the original
+    length: lo = max(floor(turn(fast)), 0), hi = min(ceil(turn(slow)), rotary_dim - 1),
+    ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1); the frequency used is f_i / factor * ramp_i + f_i * (1 - ramp_i),
+    and cosines and sines are multiplied by 0.1 ln(factor) + 1 (`magnitude`)."""
+    head_dim: int
+    theta: float
+    factor: float
+    original: float
+    fast: float
+    slow: float
+    rotary_dim: Optional[int] = None
+    pairing: str = "interleaved"
+    kind: str = "rope_scaled"
+
+    def __post_init__(self):
+        rd = self.head_dim if self.rotary_dim is None else self.rotary_dim
+        if rd <= 0 or rd % 2 or rd > self.head_dim:
+            raise ConfigError(f"rotary_dim {rd} must be even and in (0, head_dim={self.head_dim}]")
+        if not self.theta > 1:
+            raise ConfigError(f"rope theta must be above 1, got {self.theta}")
+        if not (self.factor > 0 and self.original > 0 and self.fast > 0 and self.slow > 0):
+            raise ConfigError("rope scaling: factor, original, fast and slow must be positive")
+        if self.pairing not in ("half", "interleaved"):
+            raise ConfigError(f"rope pairing {self.pairing!r} is not one of half, interleaved")
+
+
+@dataclass(frozen=True)
 class NoPositionSpec:
     """No position encoding inside the mixer."""
     kind: str = "none"
@@ -78,6 +109,13 @@ class AttentionSpec:
     `scale` None means 1/sqrt(head_dim).  `page_size` None keeps its keys in pages
     of the engine's size; P asks for pages of P tokens (a short window is served
     better by small pages), in a pool of their own.
+
+    `bias`: q, k and v have biases (`bias_names`).  `qk_norm_weight` False: the per-head norm
+    divides by the root mean square alone (no weight tensors).  `q_temp` (coef, every): the
+    query at position p is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1).
+    `v_head_dim` D: values have D numbers a head (None: as keys).  `own_kv` False: the mixer
+    has no key and value projections and reads the cache of another run (`LayerRun.cache_of`).
+    `names`: local tensor names of (q, k, v, o, q norm, k norm).
     """
     hidden_size: int
     num_heads: int
@@ -90,10 +128,23 @@ class AttentionSpec:
     prefix: str = ""
     kind: str = "attention"
     page_size: Optional[int] = None
+    bias: bool = False
+    qk_norm_weight: bool = True
+    q_temp: Optional[Tuple[float, int]] = None
+    v_head_dim: Optional[int] = None
+    own_kv: bool = True
+    names: Tuple[str, ...] = ("q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight", "q_norm.weight", "k_norm.weight")
+    bias_names: Tuple[str, str, str] = ("q_proj.bias", "k_proj.bias", "v_proj.bias")
 
     def __post_init__(self):
         if self.num_heads <= 0 or self.num_kv_heads <= 0:
             raise ConfigError("attention needs at least one query head and one key/value head")
+        if self.v_head_dim is not None and not 0 < self.v_head_dim <= 256:
+            raise ConfigError(f"value head size {self.v_head_dim} unsupported: from 1 to 256")
+        if self.q_temp is not None and not (len(self.q_temp) == 2 and isinstance(self.q_temp[1], int) and self.q_temp[1] > 0):
+            raise ConfigError("q_temp is (coef, every) with a positive integer `every`")
+        if len(self.names) != 6 or len(self.bias_names) != 3:
+            raise ConfigError("names: six local tensor names; bias_names: three")
         if self.num_heads % self.num_kv_heads:
             raise ConfigError(
                 f"num_attention_heads {self.num_heads} is not a multiple of "
@@ -115,6 +166,116 @@ class AttentionSpec:
     @property
     def kv_dim(self) -> int:
         return self.num_kv_heads * self.head_dim
+
+    @property
+    def value_dim(self) -> int:
+        return self.head_dim if self.v_head_dim is None else self.v_head_dim
+
+    @property
+    def v_dim(self) -> int:
+        return self.num_kv_heads * self.value_dim
+
+    @property
+    def out_dim(self) -> int:
+        return self.num_heads * self.value_dim
+
+    @property
+    def plain(self) -> bool:
+        """None of the extras: the mixer's first kernels (weighted norm, rotation, fused decode) apply."""
+        return not self.bias and self.qk_norm_weight and self.q_temp is None and self.v_head_dim is None and self.own_kv
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Attention whose keys and values are made from a latent of `kv_rank` numbers a token, which is all the cache keeps
+    (beside `rot_dim` numbers of a rotated key part that every head shares).
+
+    cq = N(W_dq x), q = W_uq cq, a head being [head_dim unrotated | rot_dim rotated];  W_dkv x = [c' | kr], c = N(c');
+    head h: key [W_uk_h c | rot(kr)], value W_uv_h c (`v_head_dim` numbers); score = scale * q_h . key_h; position i
+    sees j when 0 <= i - j < `window` (None: every j <= i); with `output_gate` head h's result is multiplied by
+    sigmoid(W_g x)_h.  N is an RMS norm with a plain weight and `norm_eps`.  `position` rotates the first
+    rotary_dim numbers of the rotated parts.  `names`: local tensor names of (dq, dq norm, uq, dkv, dkv norm, uk, uv, g, o)."""
+    hidden_size: int
+    num_heads: int
+    head_dim: int
+    rot_dim: int
+    v_head_dim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    norm_eps: float
+    position: object = NoPositionSpec()
+    window: Optional[int] = None
+    output_gate: bool = True
+    prefix: str = ""
+    kind: str = "latent_attention"
+    page_size: Optional[int] = None
+    names: Tuple[str, ...] = ("dq", "dq.norm", "uq", "dkv", "dkv.norm", "uk", "uv", "g", "o")
+
+    def __post_init__(self):
+        for what, v in (("heads", self.num_heads), ("head_dim", self.head_dim), ("v_head_dim", self.v_head_dim),
+                        ("q_rank", self.q_rank), ("kv_rank", self.kv_rank)):
+            if v <= 0:
+                raise ConfigError(f"latent attention: {what} must be positive, got {v}")
+        if self.rot_dim < 0:
+            raise ConfigError(f"latent attention: rot_dim must not be negative, got {self.rot_dim}")
+        if self.kv_rank + self.rot_dim > 1024 or self.head_dim > 2048 or self.kv_rank > 2048:
+            raise ConfigError("latent attention: the cached row (kv_rank + rot_dim) takes up to 1,024 numbers, head_dim and kv_rank up to 2,048")
+        if self.window is not None and self.window <= 0:
+            raise ConfigError(f"attention window must be positive, got {self.window}")
+        if len(self.names) != 9:
+            raise ConfigError("names: nine local tensor names")
+
+    @property
+    def row(self) -> int:
+        """Numbers a token keeps in the cache."""
+        return self.kv_rank + self.rot_dim
+
+
+@dataclass(frozen=True)
+class MLSTMSpec:
+    """The matrix memory of xLSTM (mLSTM): per head a state S [head_dim, v_head_dim], n [head_dim] and a running maximum m
+    of the gates' logarithms, all starting at zero, carried from token to token in float32.
+
+    q = W_q x / sqrt(head_dim), k = W_k x, v = W_v x;  li = cap tanh((W_i x + b_i) / cap),
+    lf = logsigmoid(cap tanh((W_f x + b_f) / cap)), cap = `gate_cap`;  m' = max(lf + m, li);
+    S' = e^(lf + m - m') S + e^(li - m') k v^T, n' likewise with k;  o = S'^T q / (max(|n' . q|, e^(-m')) + 1e-6);
+    every head of o over its root mean square (`norm_eps`), times the norm weight, times sigmoid(W_g x), then W_o.
+    `names`: local tensor names of (q, k, v, g, o, norm, i, i bias, f, f bias)."""
+    hidden_size: int
+    num_heads: int
+    head_dim: int
+    v_head_dim: int
+    gate_cap: float
+    norm_eps: float
+    prefix: str = ""
+    kind: str = "mlstm"
+    names: Tuple[str, ...] = ("q", "k", "v", "g", "o", "norm", "i", "i.b", "f", "f.b")
+
+    def __post_init__(self):
+        if self.num_heads <= 0 or self.v_head_dim <= 0 or not 0 < self.head_dim <= 256:
+            raise ConfigError("mlstm: heads and value size must be positive, key size from 1 to 256")
+        if not self.gate_cap > 0:
+            raise ConfigError(f"mlstm: gate_cap must be positive, got {self.gate_cap}")
+        if len(self.names) != 10:
+            raise ConfigError("names: ten local tensor names")
+
+
+@dataclass(frozen=True)
+class HyperConnectionSpec:
+    """How one sublayer reads from and writes to `streams` copies of the residual stream: it reads sum_r in[r] X_r and
+    its result y goes back as X_t <- sum_r mix[r, t] X_r + out[t] y for every t at once.  `learned` False: no tensors,
+    every coefficient is one where it is on the diagonal or a vector (one copy is then the plain residual sum).
+    `names`: local tensor names of (in, out, mix)."""
+    streams: int
+    prefix: str = ""
+    learned: bool = True
+    kind: str = "hyper"
+    names: Tuple[str, str, str] = ("in", "out", "mix")
+
+    def __post_init__(self):
+        if not 0 < self.streams <= 8:
+            raise ConfigError(f"streams must be from 1 to 8, got {self.streams}")
 
 
 @dataclass(frozen=True)
@@ -205,7 +366,10 @@ class LayerSpec:
     and computes x += mixer(mixer_norm(x)); x += ffn(ffn_norm(x)).  The "post_norm"
     arrangement has the same roles and norms after the sum, the sublayers reading x
     itself: x = mixer_norm(a x + mixer(x)); x = ffn_norm(a x + ffn(x)) with
-    a = `residual_scale`; "post_norm_mixer" is its first half alone.
+    a = `residual_scale`; "post_norm_mixer" is its first half alone.  "hyper_pre_norm" keeps
+    several copies of the residual stream and has the roles mixer_norm, mixer_hc, mixer,
+    ffn_norm, ffn_hc, ffn (the *_hc parts say how a sublayer reads and writes the copies);
+    "hyper_pre_norm_mixer" is its first half alone.
     """
     parts: Tuple[Tuple[str, object], ...]
     block: str = "pre_norm"
@@ -244,12 +408,14 @@ class EmbeddingSpec:
 
 @dataclass(frozen=True)
 class HeadSpec:
-    """Output head: logits = W x.  `tied` aliases the embedding table."""
+    """Output head: logits = W x * scale.  `tied` aliases the embedding table; else the tensor is prefix + name."""
     vocab_size: int
     hidden_size: int
     tied: bool
     prefix: str = "lm_head."
     kind: str = "lm_head"
+    scale: float = 1.0
+    name: str = "weight"
 
 
 @dataclass(frozen=True)
@@ -265,8 +431,12 @@ class ModelSpec:
     head: HeadSpec
     stop_tokens: Tuple[int, ...] = field(default_factory=tuple)
     input_position: Optional[object] = None   # a position part applied to the residual stream after the embedding (None: none)
+    streams: Optional[int] = None             # copies of the residual stream (None: one row a token; every layer is then no "hyper" block)
 
     def __post_init__(self):
+        hyper = [layer.block.startswith("hyper_") for layer in self.layers]
+        if any(hyper) != (self.streams is not None) or (any(hyper) and not all(hyper)):
+            raise ConfigError("a model keeps several copies of the residual stream in every layer or in none")
         for index, run in enumerate(self.order):
             if not 0 <= run.layer < len(self.layers):
                 raise ConfigError(f"order[{index}] names layer {run.layer} of {len(self.layers)}")

@@ -1,6 +1,8 @@
 // Causal grouped-query attention over the paged cache for any mix of query
-// tokens (prompt portions and single decoded tokens alike), any head size up
-// to 256 and any storage type.  One wave per (token, query head); this is the
+// tokens (prompt portions and single decoded tokens alike), any key size up
+// to 1,024, values of their own width (`dv`; the value cache may be the key
+// cache itself, a value then being the first dv numbers of its key's row of
+// `v_row` numbers) and any storage type.  One wave per (token, query head); this is the
 // float32 path's kernel and the fallback of sizes the MFMA kernels refuse.
 //
 // For query position p of a sequence the keys are s in [max(0, p-window+1), p]
@@ -13,14 +15,14 @@
 #include <math.h>
 
 #define HEADS_PER_BLOCK 4
-#define MAX_D 256
+#define MAX_D 1024
 
 template <typename TQ, typename TC, typename TO>
 __global__ void paged_attention_generic_kernel(
     const TQ* __restrict__ q, const TC* __restrict__ k_cache, const TC* __restrict__ v_cache, TO* __restrict__ out,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
     const int32_t* __restrict__ block_table, int max_blocks,
-    int n_q, int n_kv, int d, int page, float scale, int window) {
+    int n_q, int n_kv, int d, int dv, int v_row, int page, float scale, int window) {
     __shared__ float q_s[HEADS_PER_BLOCK][MAX_D];
     __shared__ float p_s[HEADS_PER_BLOCK][KIPP_WAVE];
     __shared__ unsigned long long off_s[HEADS_PER_BLOCK][KIPP_WAVE];
@@ -52,8 +54,8 @@ __global__ void paged_attention_generic_kernel(
         unsigned long long off = 0;
         if (valid) {
             const int page_id = table[s / page];
-            off = (((unsigned long long)page_id * n_kv + g) * page + s % page) * d;
-            const TC* k_row = k_cache + off;
+            off = ((unsigned long long)page_id * n_kv + g) * page + s % page;
+            const TC* k_row = k_cache + off * d;
             float dot = 0.0f;
             for (int e = 0; e < d; ++e) dot += q_s[wave][e] * load_f(k_row, e);
             score = dot * scale;
@@ -72,37 +74,47 @@ __global__ void paged_attention_generic_kernel(
 #pragma unroll
         for (int c = 0; c < MAX_D / KIPP_WAVE; ++c) {
             const int e = lane + c * KIPP_WAVE;
-            if (e < d) {
+            if (e < dv) {
                 float a = acc[c] * alpha;
-                for (int j = j_lo; j < j_hi; ++j) a += p_s[wave][j] * load_f(v_cache + off_s[wave][j], e);
+                for (int j = j_lo; j < j_hi; ++j) a += p_s[wave][j] * load_f(v_cache + off_s[wave][j] * v_row, e);
                 acc[c] = a;
             }
         }
     }
     if (!active) return;
-    TO* o_row = out + ((size_t)t * n_q + head) * d;
+    TO* o_row = out + ((size_t)t * n_q + head) * dv;
     const float inv = 1.0f / l;
 #pragma unroll
     for (int c = 0; c < MAX_D / KIPP_WAVE; ++c) {
         const int e = lane + c * KIPP_WAVE;
-        if (e < d) store_f(o_row, e, acc[c] * inv);
+        if (e < dv) store_f(o_row, e, acc[c] * inv);
     }
+}
+
+// Values of width dv in rows of v_row numbers (v_row = dv for a value cache of its own).
+extern "C" int kipp_paged_attention_generic_v(
+    const void* q, int q_dtype, const void* k_cache, const void* v_cache, int cache_dtype, void* out, int out_dtype,
+    const int32_t* positions, const int32_t* seq_of_token, const int32_t* block_table, int max_blocks,
+    int n_tokens, int n_q, int n_kv, int d, int dv, int v_row, int page, float scale, int window, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (d > MAX_D || d <= 0 || dv > MAX_D || dv <= 0 || v_row < dv || n_kv <= 0 || n_q % n_kv) return -1;
+    dim3 grid((n_q + HEADS_PER_BLOCK - 1) / HEADS_PER_BLOCK, n_tokens), block(HEADS_PER_BLOCK * KIPP_WAVE);
+#define KIPP_PA(TQ, TC, TO)                                                                                    \
+    hipLaunchKernelGGL((paged_attention_generic_kernel<TQ, TC, TO>), grid, block, 0, stream, (const TQ*)q,     \
+                       (const TC*)k_cache, (const TC*)v_cache, (TO*)out, positions, seq_of_token, block_table, \
+                       max_blocks, n_q, n_kv, d, dv, v_row, page, scale, window)
+    if (q_dtype == KIPP_F32 && cache_dtype == KIPP_F32 && out_dtype == KIPP_F32) KIPP_PA(float, float, float);
+    else if (q_dtype == KIPP_BF16 && cache_dtype == KIPP_BF16 && out_dtype == KIPP_BF16) KIPP_PA(bf16_t, bf16_t, bf16_t);
+    else return -2;
+#undef KIPP_PA
+    return KIPP_LAUNCH_CHECK();
 }
 
 extern "C" int kipp_paged_attention_generic(
     const void* q, int q_dtype, const void* k_cache, const void* v_cache, int cache_dtype, void* out, int out_dtype,
     const int32_t* positions, const int32_t* seq_of_token, const int32_t* block_table, int max_blocks,
     int n_tokens, int n_q, int n_kv, int d, int page, float scale, int window, hipStream_t stream) {
-    if (n_tokens <= 0) return 0;
-    if (d > MAX_D || d <= 0 || n_kv <= 0 || n_q % n_kv) return -1;
-    dim3 grid((n_q + HEADS_PER_BLOCK - 1) / HEADS_PER_BLOCK, n_tokens), block(HEADS_PER_BLOCK * KIPP_WAVE);
-#define KIPP_PA(TQ, TC, TO)                                                                                    \
-    hipLaunchKernelGGL((paged_attention_generic_kernel<TQ, TC, TO>), grid, block, 0, stream, (const TQ*)q,     \
-                       (const TC*)k_cache, (const TC*)v_cache, (TO*)out, positions, seq_of_token, block_table, \
-                       max_blocks, n_q, n_kv, d, page, scale, window)
-    if (q_dtype == KIPP_F32 && cache_dtype == KIPP_F32 && out_dtype == KIPP_F32) KIPP_PA(float, float, float);
-    else if (q_dtype == KIPP_BF16 && cache_dtype == KIPP_BF16 && out_dtype == KIPP_BF16) KIPP_PA(bf16_t, bf16_t, bf16_t);
-    else return -2;
-#undef KIPP_PA
-    return KIPP_LAUNCH_CHECK();
+    if (d > 256) return -1;
+    return kipp_paged_attention_generic_v(q, q_dtype, k_cache, v_cache, cache_dtype, out, out_dtype, positions, seq_of_token,
+                                          block_table, max_blocks, n_tokens, n_q, n_kv, d, d, d, page, scale, window, stream);
 }

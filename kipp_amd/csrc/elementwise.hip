@@ -417,6 +417,11 @@ static void launch_rmsnorm(float* x, const void* delta, const float* weight, voi
     }
 }
 
+// x[i] *= s, float32 (logits times a model's constant)
+__global__ void scale_values_kernel(float* __restrict__ x, float s, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) x[i] *= s;
+}
+
 extern "C" {
 
 int kipp_embed(const void* table, int table_dtype, const int32_t* tokens, float* out,
@@ -577,6 +582,13 @@ int kipp_fill_zero(void* out, size_t words, hipStream_t stream) {
     if (words == 0) return 0;
     const unsigned blocks = (unsigned)((words + 255) / 256 < 2048 ? (words + 255) / 256 : 2048);
     hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, stream, (uint32_t*)out, words);
+    return KIPP_LAUNCH_CHECK();
+}
+
+int kipp_scale_values(float* x, float s, size_t n, hipStream_t stream) {
+    if (n == 0) return 0;
+    const unsigned blocks = (unsigned)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+    hipLaunchKernelGGL(scale_values_kernel, dim3(blocks), dim3(256), 0, stream, x, s, n);
     return KIPP_LAUNCH_CHECK();
 }
 

@@ -172,6 +172,15 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor, pairs: bool = False) -> tor
     return out
 
 
+def scale_values(x: torch.Tensor, scale: float) -> torch.Tensor:
+    """x *= scale in place (float32)."""
+    _dev(x)
+    _need(x.dtype == torch.float32, "scale_values: float32")
+    fn = _fn("elementwise", "kipp_scale_values", [_c_ptr, _c_float, _c_size, _c_ptr])
+    _check(fn(_ptr(x), float(scale), x.numel(), _stream()), "scale_values")
+    return x
+
+
 def cast(src: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     _dev(src, out)
     _need(src.numel() == out.numel(), "cast: sizes differ")
@@ -306,6 +315,258 @@ def _attn_common(q, k_cache, v_cache, out, n_q, n_kv, head_dim, what):
     _need(head_dim % 16 == 0 and 0 < head_dim <= 256 and n_q % n_kv == 0, f"{what}: head size or head counts refused")
     page = k_cache.shape[2]
     _need(page > 0 and page & (page - 1) == 0, f"{what}: the page size must be a power of two (the generic kernel takes any)")
+
+
+# --------------------------------------------------------------------------- several residual streams
+
+STREAMS_MAX = 8
+
+
+def streams_open(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out [tokens, R, width] (float32): every one of the R rows of a token is table[token]."""
+    _dev(table, tokens, out)
+    _i32(tokens, "tokens")
+    _need(out.dim() == 3 and out.dtype == torch.float32 and table.dim() == 2 and table.shape[1] == out.shape[2]
+          and tokens.numel() == out.shape[0] and 0 < out.shape[1] <= STREAMS_MAX, "streams_open: out is float32 [tokens, R <= 8, width]")
+    fn = _fn("streams", "kipp_streams_open", [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(table), _code(table), _ptr(tokens), _ptr(out), out.shape[0], out.shape[1], out.shape[2], _stream()), "streams_open")
+    return out
+
+
+def _streams_write_args(x, delta, mix, outw, what):
+    n, r, width = x.shape
+    parts = 0
+    if delta is not None:
+        _need(delta.dtype == torch.float32 and delta.dim() in (2, 3) and tuple(delta.shape[-2:]) == (n, width),
+              f"{what}: delta is float32 [tokens, width] or slabs of it")
+        parts = delta.shape[0] if delta.dim() == 3 else 1
+        _need(mix is not None and outw is not None and mix.dtype == outw.dtype == torch.float32 and mix.numel() == r * r
+              and outw.numel() == r, f"{what}: float32 coefficients [R, R] and [R]")
+    else:
+        _need(mix is None and outw is None, f"{what}: coefficients without a delta")
+    return parts
+
+
+def streams_step(x: torch.Tensor, delta: Optional[torch.Tensor], mix: Optional[torch.Tensor], outw: Optional[torch.Tensor],
+                 inw: Optional[torch.Tensor], norm_w: Optional[torch.Tensor], eps: float, h: Optional[torch.Tensor]):
+    """One pass over the R rows of every token of x [tokens, R, width] (float32): with `delta` (a sublayer's result,
+    maybe in slabs) the rows become X_t <- sum_r mix[r, t] X_r + outw[t] delta; with `inw` the weighted sum
+    sum_r inw[r] X_r is RMS-normed with `norm_w` into `h` [tokens, width]."""
+    _dev(x, delta, mix, outw, inw, norm_w, h)
+    _need(x.dim() == 3 and x.dtype == torch.float32 and 0 < x.shape[1] <= STREAMS_MAX, "streams_step: x is float32 [tokens, R <= 8, width]")
+    n, r, width = x.shape
+    parts = _streams_write_args(x, delta, mix, outw, "streams_step")
+    if inw is not None:
+        _need(inw.dtype == torch.float32 and inw.numel() == r and norm_w is not None and norm_w.dtype == torch.float32
+              and norm_w.numel() == width and h is not None and h.shape == (n, width), "streams_step: float32 [R] and [width], h [tokens, width]")
+    _need(delta is not None or inw is not None, "streams_step: nothing to do")
+    fn = _fn("streams", "kipp_streams_step", [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_int,
+                                              _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), _ptr(delta), parts, _ptr(mix), _ptr(outw), _ptr(inw), _ptr(norm_w), float(eps),
+              _ptr(h) if inw is not None else None, _code(h) if inw is not None else F32, n, r, width, _stream()), "streams_step")
+    return h
+
+
+def streams_close(x: torch.Tensor, delta: Optional[torch.Tensor], mix: Optional[torch.Tensor], outw: Optional[torch.Tensor],
+                  which: Optional[torch.Tensor], out: torch.Tensor) -> torch.Tensor:
+    """out [rows, width] (float32) = the sum of a token's R rows after the last write (which is not stored), for the
+    tokens that `which` names (None: all, in order)."""
+    _dev(x, delta, mix, outw, which, out)
+    _need(x.dim() == 3 and x.dtype == torch.float32 and 0 < x.shape[1] <= STREAMS_MAX, "streams_close: x is float32 [tokens, R <= 8, width]")
+    n, r, width = x.shape
+    parts = _streams_write_args(x, delta, mix, outw, "streams_close")
+    if which is not None:
+        _i32(which, "which")
+    rows = which.numel() if which is not None else n
+    _need(out.dtype == torch.float32 and out.shape == (rows, width), "streams_close: out is float32 [rows, width]")
+    fn = _fn("streams", "kipp_streams_close", [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), _ptr(delta), parts, _ptr(mix), _ptr(outw), _ptr(which), _ptr(out), n, rows, r, width, _stream()), "streams_close")
+    return out
+
+
+# --------------------------------------------------------------------------- heads made ready without a rotation
+
+def head_prepare(proj: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                 positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
+                 n_q: int, n_kv: int, d: int, dv: int, bias: Optional[torch.Tensor], norm: str, eps: float,
+                 q_norm_w: Optional[torch.Tensor] = None, k_norm_w: Optional[torch.Tensor] = None,
+                 temp_coef: float = 0.0, temp_every: int = 0, write_kv: bool = True) -> torch.Tensor:
+    """From a step's input product `proj` (float32 [tokens, >= n_q d + n_kv d + n_kv dv], columns q | k | v | ..., or slabs
+    of it): `bias` added (float32 over the q | k | v columns), every head of q and k RMS-normed (`norm`: "none", "plain"
+    or "weighted" with `q_norm_w` / `k_norm_w` [d]), queries at position p times 1 + temp_coef ln(floor((p + 1) /
+    temp_every) + 1) (temp_every 0: none), q kept in `q_out`, k and v written into the pages of their positions."""
+    _dev(proj, q_out, k_cache, v_cache, positions, seq_of_token, block_table, bias, q_norm_w, k_norm_w)
+    for t, name in ((positions, "positions"), (seq_of_token, "seq_of_token"), (block_table, "block_table")):
+        _i32(t, name)
+    parts, n, stride = _slabs(proj, "head_prepare")
+    _need(norm in ("none", "plain", "weighted"), "head_prepare: norm is one of none, plain, weighted")
+    _need(stride >= n_q * d + (n_kv * d + n_kv * dv if write_kv else 0), "head_prepare: the projections are narrower than q, k and v")
+    _need(0 < d <= 256 and 0 < dv <= 256, "head_prepare: head sizes from 1 to 256")
+    _need(q_out.shape == (n, n_q * d) and positions.numel() == n and seq_of_token.numel() == n, "head_prepare: one row a token")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.numel() == n_q * d + n_kv * d + n_kv * dv, "head_prepare: float32 bias over q | k | v")
+    if norm == "weighted":
+        _need(q_norm_w is not None and k_norm_w is not None and q_norm_w.dtype == k_norm_w.dtype == torch.float32
+              and q_norm_w.numel() == d and k_norm_w.numel() == d, "head_prepare: float32 norm weights [d]")
+    _need(k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.shape[:3] == v_cache.shape[:3] and k_cache.shape[1] == n_kv
+          and k_cache.shape[3] == d and v_cache.shape[3] == dv and k_cache.dtype == v_cache.dtype,
+          "head_prepare: caches must be [pages, n_kv, page, d] and [pages, n_kv, page, dv]")
+    _need(block_table.dim() == 2 and int(temp_every) >= 0, "head_prepare: block_table is [sequences, blocks]")
+    fn = _fn("head_prepare", "kipp_head_prepare",
+             [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
+              _c_int, _c_ptr, _c_ptr, _c_float, _c_float, _c_int] + [_c_int] * 7 + [_c_ptr])
+    _check(fn(_ptr(proj), parts, stride, _ptr(bias), _ptr(q_out), _code(q_out), _ptr(k_cache), _ptr(v_cache), _code(k_cache),
+              _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1],
+              {"none": 0, "plain": 1, "weighted": 2}[norm], _ptr(q_norm_w), _ptr(k_norm_w), float(eps), float(temp_coef),
+              int(temp_every), n, n_q, n_kv, d, dv, k_cache.shape[2], int(write_kv), _stream()), "head_prepare")
+    return q_out
+
+
+def paged_attention_wide(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
+                         positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
+                         n_q: int, n_kv: int, d: int, dv: int, scale: float, window: int = 0) -> torch.Tensor:
+    """The generic attention kernel with values of their own width: keys of up to 1,024 numbers, values of `dv`.
+    `v_cache` may be `k_cache` itself: a value is then the first dv numbers of its key's row."""
+    _dev(q, k_cache, v_cache, out, positions, seq_of_token, block_table)
+    for t, name in ((positions, "positions"), (seq_of_token, "seq_of_token"), (block_table, "block_table")):
+        _i32(t, name)
+    n = q.shape[0]
+    _need(q.shape == (n, n_q * d) and out.shape == (n, n_q * dv), "attention: q is [tokens, n_q d] and out [tokens, n_q dv]")
+    _need(k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.shape[:3] == v_cache.shape[:3] and k_cache.shape[1] == n_kv
+          and k_cache.shape[3] == d and v_cache.shape[3] >= dv and k_cache.dtype == v_cache.dtype and 0 < d <= 1024 and 0 < dv <= 1024,
+          "attention: caches must be [pages, n_kv, page, d] and [pages, n_kv, page, >= dv] of one type")
+    _need(positions.numel() == n and seq_of_token.numel() == n and block_table.dim() == 2,
+          "attention: one position and sequence per token, block_table [sequences, blocks]")
+    fn = _fn("attention_generic", "kipp_paged_attention_generic_v",
+             [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
+              _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr])
+    _check(fn(_ptr(q), _code(q), _ptr(k_cache), _ptr(v_cache), _code(k_cache), _ptr(out), _code(out),
+              _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1],
+              n, n_q, n_kv, d, dv, v_cache.shape[3], k_cache.shape[2], float(scale), int(window), _stream()),
+           "paged_attention_wide")
+    return out
+
+
+# --------------------------------------------------------------------------- attention through a latent
+
+def latent_prepare(proj: torch.Tensor, cq_out: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor,
+                   seq_of_token: torch.Tensor, block_table: torch.Tensor, q_rank: int, rank: int, dr: int,
+                   q_norm_w: torch.Tensor, c_norm_w: torch.Tensor, eps: float, freq: torch.Tensor, rot_dims: int,
+                   magnitude: float, write_kv: bool = True) -> torch.Tensor:
+    """From the input product `proj` (float32 [tokens, >= q_rank + rank + dr], columns query latent | key/value latent |
+    rotated key part | ..., or slabs of it): the query latent RMS-normed with `q_norm_w` into `cq_out`; the key/value latent
+    RMS-normed with `c_norm_w` and the key part rotated at the token's position, both written as one row of rank + dr
+    numbers into the token's page of `cache` [pages, 1, page, rank + dr]."""
+    _dev(proj, cq_out, cache, positions, seq_of_token, block_table, q_norm_w, c_norm_w, freq)
+    for t, name in ((positions, "positions"), (seq_of_token, "seq_of_token"), (block_table, "block_table")):
+        _i32(t, name)
+    parts, n, stride = _slabs(proj, "latent_prepare")
+    _need(stride >= q_rank + rank + dr and cq_out.shape == (n, q_rank) and positions.numel() == n and seq_of_token.numel() == n,
+          "latent_prepare: one row a token, projections [query latent | latent | rotated part]")
+    _need(cache.dim() == 4 and cache.shape[1] == 1 and cache.shape[3] == rank + dr and block_table.dim() == 2,
+          "latent_prepare: the cache is [pages, 1, page, rank + dr]")
+    _need(q_norm_w.dtype == c_norm_w.dtype == torch.float32 and q_norm_w.numel() == q_rank and c_norm_w.numel() == rank,
+          "latent_prepare: float32 norm weights")
+    _need(rot_dims % 2 == 0 and 0 <= rot_dims <= dr and freq.dtype == torch.float32 and freq.numel() >= rot_dims // 2,
+          "latent_prepare: float32 frequencies for rot_dims / 2 pairs")
+    fn = _fn("latent", "kipp_latent_prepare",
+             [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
+              _c_ptr, _c_int, _c_float] + [_c_int] * 6 + [_c_ptr])
+    _check(fn(_ptr(proj), parts, stride, _ptr(q_norm_w), _ptr(c_norm_w), float(eps), _ptr(cq_out), _code(cq_out), _ptr(cache),
+              _code(cache), _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1], _ptr(freq), int(rot_dims),
+              float(magnitude), n, q_rank, rank, dr, cache.shape[2], int(write_kv), _stream()), "latent_prepare")
+    return cq_out
+
+
+def latent_absorb(q: torch.Tensor, w_uk: torch.Tensor, out: torch.Tensor, positions: torch.Tensor, freq: torch.Tensor,
+                  rot_dims: int, magnitude: float, heads: int, d: int, dr: int, rank: int) -> torch.Tensor:
+    """out [tokens, heads (rank + dr)]: every head's unrotated query part carried into the latent's space by
+    `w_uk` [heads d, rank] (q_h W_uk_h), its rotated part turned at the token's position."""
+    _dev(q, w_uk, out, positions, freq)
+    _i32(positions, "positions")
+    parts, n, stride = _slabs(q, "latent_absorb")
+    _need(stride == heads * (d + dr) and out.shape == (n, heads * (rank + dr)) and positions.numel() == n,
+          "latent_absorb: q is [tokens, heads (d + dr)], out [tokens, heads (rank + dr)]")
+    _need(w_uk.shape == (heads * d, rank) and _code(w_uk) == _code(out), "latent_absorb: w_uk is [heads d, rank] in the output's type")
+    _need(d * 32 <= 64 * 1024, "latent_absorb: unrotated head size too large")
+    fn = _fn("latent", "kipp_latent_absorb", [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_float]
+             + [_c_int] * 5 + [_c_ptr])
+    _check(fn(_ptr(q), parts, _ptr(w_uk), _code(w_uk), _ptr(out), _code(out), _ptr(positions), _ptr(freq), int(rot_dims),
+              float(magnitude), n, heads, d, dr, rank, _stream()), "latent_absorb")
+    return out
+
+
+def latent_expand(lat: torch.Tensor, w_uv_t: torch.Tensor, out: torch.Tensor, heads: int, rank: int, dv: int,
+                  gate: Optional[torch.Tensor] = None, gate_at: int = 0) -> torch.Tensor:
+    """out [tokens, heads dv]: head h's latent result (the first `rank` numbers of its row of `lat` [tokens, heads row])
+    carried back by `w_uv_t` [heads, rank, dv], times sigmoid(gate[t, gate_at + h]) where `gate` (the float32 input
+    product, maybe in slabs) is given."""
+    _dev(lat, w_uv_t, out, gate)
+    n = lat.shape[0]
+    _need(lat.dim() == 2 and lat.shape[1] % heads == 0 and lat.shape[1] // heads >= rank, "latent_expand: lat is [tokens, heads row]")
+    _need(w_uv_t.shape == (heads, rank, dv) and out.shape == (n, heads * dv) and _code(lat) == _code(w_uv_t) == _code(out),
+          "latent_expand: w_uv_t is [heads, rank, dv]; one type")
+    _need(rank * 32 <= 64 * 1024, "latent_expand: latent too wide")
+    g_parts, g_stride, g_ptr = 0, 0, None
+    if gate is not None:
+        g_parts, g_n, g_stride = _slabs(gate, "latent_expand")
+        _need(g_n == n and gate_at + heads <= g_stride, "latent_expand: the gate's columns lie outside the product")
+        g_ptr = gate.data_ptr() + 4 * gate_at
+    fn = _fn("latent", "kipp_latent_expand", [_c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr, _c_int]
+             + [_c_int] * 4 + [_c_ptr])
+    _check(fn(_ptr(lat), _code(lat), lat.shape[1] // heads, _ptr(w_uv_t), _code(w_uv_t), g_ptr, g_parts, g_stride, _ptr(out),
+              _code(out), n, heads, rank, dv, _stream()), "latent_expand")
+    return out
+
+
+# --------------------------------------------------------------------------- matrix memory (mLSTM)
+
+MLSTM_COLS = 64     # columns of the memory a workgroup of the scan takes
+
+
+def mlstm_state_size(heads: int, d: int, dv: int) -> int:
+    """float32 numbers of a request's state: S [heads, d, dv], then a copy of n [heads, d] and m [heads] for every
+    MLSTM_COLS columns."""
+    return heads * d * dv + -(-dv // MLSTM_COLS) * (heads * d + heads)
+
+
+def mlstm_scan(proj: torch.Tensor, bias_i: torch.Tensor, bias_f: torch.Tensor, cap: float, state: torch.Tensor,
+               q_start: torch.Tensor, q_len: torch.Tensor, slots: torch.Tensor, o_raw: torch.Tensor,
+               heads: int, d: int, dv: int) -> torch.Tensor:
+    """The recurrence over every entry's tokens, in order, from and into the entry's slot of `state` [slots, size]
+    (float32).  `proj`: float32 [tokens, >= 2 heads d + 2 heads dv + 2 heads], columns q | k | v | gate | zi | zf;
+    `o_raw` float32 [tokens, heads dv] receives S^T q over its denominator."""
+    _dev(proj, bias_i, bias_f, state, q_start, q_len, slots, o_raw)
+    for t, name in ((q_start, "q_start"), (q_len, "q_len"), (slots, "slots")):
+        _i32(t, name)
+    _need(proj.dim() == 2 and proj.dtype == torch.float32 and proj.shape[1] >= 2 * heads * d + 2 * heads * dv + 2 * heads,
+          "mlstm_scan: proj is float32 [tokens, q | k | v | gate | zi | zf]")
+    _need(state.dim() == 2 and state.dtype == torch.float32 and state.shape[1] >= mlstm_state_size(heads, d, dv),
+          "mlstm_scan: state is float32 [slots, size]")
+    _need(bias_i.dtype == bias_f.dtype == torch.float32 and bias_i.numel() == heads and bias_f.numel() == heads, "mlstm_scan: float32 gate biases [heads]")
+    _need(o_raw.dtype == torch.float32 and o_raw.shape == (proj.shape[0], heads * dv) and 0 < d <= 256 and cap > 0,
+          "mlstm_scan: o_raw is float32 [tokens, heads dv]; key size up to 256")
+    _need(q_start.numel() == q_len.numel() == slots.numel(), "mlstm_scan: one start, length and slot an entry")
+    fn = _fn("mlstm", "kipp_mlstm_scan", [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_size, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                                          _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(proj), proj.shape[1], _ptr(bias_i), _ptr(bias_f), float(cap), _ptr(state), state.shape[1], _ptr(q_start),
+              _ptr(q_len), _ptr(slots), _ptr(o_raw), q_start.numel(), heads, d, dv, _stream()), "mlstm_scan")
+    return o_raw
+
+
+def mlstm_finish(o_raw: torch.Tensor, proj: torch.Tensor, gate_at: int, norm_w: torch.Tensor, eps: float, out: torch.Tensor,
+                 heads: int, dv: int) -> torch.Tensor:
+    """out [tokens, heads dv] = every head of `o_raw` over its root mean square, times `norm_w`, times
+    sigmoid(proj[:, gate_at:gate_at + heads dv])."""
+    _dev(o_raw, proj, norm_w, out)
+    n = o_raw.shape[0]
+    _need(o_raw.dtype == proj.dtype == norm_w.dtype == torch.float32 and o_raw.shape == (n, heads * dv) and out.shape == o_raw.shape
+          and proj.dim() == 2 and proj.shape[0] == n and proj.shape[1] >= gate_at + heads * dv and norm_w.numel() == heads * dv,
+          "mlstm_finish: float32 [tokens, heads dv] rows, gate columns inside proj")
+    fn = _fn("mlstm", "kipp_mlstm_finish", [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_float, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(o_raw), _ptr(proj), proj.shape[1], int(gate_at), _ptr(norm_w), float(eps), _ptr(out), _code(out), n, heads, dv,
+              _stream()), "mlstm_finish")
+    return out
 
 
 # --------------------------------------------------------------------------- attention with mixed heads

@@ -1,0 +1,179 @@
+// Several copies of the residual stream ("hyper-connections").
+//
+// Instead of one row x a token there are R rows X_1 .. X_R, kept as float32 [tokens][R][width].  A sublayer
+// reads a weighted sum of them and its result y goes back into all of them at once:
+//
+//     read    u = sum_r a[r] X_r ;  h = u * rsqrt(mean(u^2) + eps) * w          (the sublayer's RMS norm)
+//     write   X_t <- sum_r M[r][t] X_r + b[t] y       for every t, from the old rows
+//
+// A layer's write and the next sublayer's read are one pass over the token's rows (`kipp_streams_step` takes
+// either half or both): the rows are read once, written once, and the normed row leaves in the type the next
+// product reads.  y may come as slabs [parts][tokens][width] of a product whose contraction was split; they
+// are added in order.  Everything is float32; a token is one workgroup's, and the sums of a token run in an
+// order that its own row fixes.
+//
+//     open    X_r = table[token] for every r
+//     close   out = sum_t (sum_r M[r][t] X_r + b[t] y), for all tokens or for the rows named by `rows`
+//             (what the final norm reads; nothing is written back)
+#include "common.h"
+
+#define STREAMS_MAX 8
+
+template <typename TT>
+__global__ void streams_open_kernel(const TT* __restrict__ table, const int32_t* __restrict__ tokens, float* __restrict__ X,
+                                    int R, int width) {
+    const int t = blockIdx.x;
+    const TT* src = table + (size_t)tokens[t] * width;
+    float* dst = X + (size_t)t * R * width;
+    for (int e = threadIdx.x; e < width; e += blockDim.x) {
+        const float v = load_f(src, e);
+        for (int r = 0; r < R; ++r) dst[(size_t)r * width + e] = v;
+    }
+}
+
+struct StreamCoefficients {
+    float mix[STREAMS_MAX][STREAMS_MAX];   // [from][to]
+    float out[STREAMS_MAX];
+    float in[STREAMS_MAX];
+};
+
+__device__ __forceinline__ void load_coefficients(StreamCoefficients& c, const float* mix, const float* outw, const float* inw, int R) {
+    for (int s = 0; s < R; ++s) {
+        for (int t = 0; t < R; ++t) c.mix[s][t] = mix != nullptr ? mix[s * R + t] : 0.0f;
+        c.out[s] = outw != nullptr ? outw[s] : 0.0f;
+        c.in[s] = inw != nullptr ? inw[s] : 0.0f;
+    }
+}
+
+// write (if mix != nullptr), then read and norm (if inw != nullptr).  LDS: width floats + 16.
+template <typename TO>
+__global__ void streams_step_kernel(float* __restrict__ X, const float* __restrict__ delta, int parts, size_t part_stride,
+                                    const float* __restrict__ mix, const float* __restrict__ outw,
+                                    const float* __restrict__ inw, const float* __restrict__ norm_w, float eps,
+                                    TO* __restrict__ h, int R, int width) {
+    extern __shared__ float lds[];
+    float* u_s = lds + 16;
+    const int t = blockIdx.x;
+    float* rows = X + (size_t)t * R * width;
+    StreamCoefficients c;
+    load_coefficients(c, mix, outw, inw, R);
+    float ss = 0.0f;
+    for (int e = threadIdx.x; e < width; e += blockDim.x) {
+        float x[STREAMS_MAX];
+#pragma unroll
+        for (int r = 0; r < STREAMS_MAX; ++r) x[r] = r < R ? rows[(size_t)r * width + e] : 0.0f;
+        if (mix != nullptr) {
+            float y = 0.0f;
+            for (int p = 0; p < parts; ++p) y += delta[p * part_stride + (size_t)t * width + e];
+            float fresh[STREAMS_MAX];
+#pragma unroll
+            for (int to = 0; to < STREAMS_MAX; ++to) {
+                float v = 0.0f;
+                if (to < R) {
+#pragma unroll
+                    for (int s = 0; s < STREAMS_MAX; ++s)
+                        if (s < R) v += c.mix[s][to] * x[s];
+                    v += c.out[to] * y;
+                    rows[(size_t)to * width + e] = v;
+                }
+                fresh[to] = v;
+            }
+#pragma unroll
+            for (int r = 0; r < STREAMS_MAX; ++r) x[r] = fresh[r];
+        }
+        if (inw != nullptr) {
+            float u = 0.0f;
+#pragma unroll
+            for (int r = 0; r < STREAMS_MAX; ++r)
+                if (r < R) u += c.in[r] * x[r];
+            u_s[e] = u;
+            ss = fmaf(u, u, ss);
+        }
+    }
+    if (inw == nullptr) return;
+    ss = block_sum(ss, lds);
+    const float scale = 1.0f / sqrtf(ss / (float)width + eps);
+    TO* dst = h + (size_t)t * width;
+    for (int e = threadIdx.x; e < width; e += blockDim.x) store_f(dst, e, u_s[e] * scale * norm_w[e]);
+}
+
+__global__ void streams_close_kernel(const float* __restrict__ X, const float* __restrict__ delta, int parts, size_t part_stride,
+                                     const float* __restrict__ mix, const float* __restrict__ outw,
+                                     const int32_t* __restrict__ which, float* __restrict__ out, int R, int width) {
+    const int i = blockIdx.x;
+    const int t = which != nullptr ? which[i] : i;
+    const float* rows = X + (size_t)t * R * width;
+    StreamCoefficients c;
+    load_coefficients(c, mix, outw, nullptr, R);
+    for (int e = threadIdx.x; e < width; e += blockDim.x) {
+        float x[STREAMS_MAX];
+#pragma unroll
+        for (int r = 0; r < STREAMS_MAX; ++r) x[r] = r < R ? rows[(size_t)r * width + e] : 0.0f;
+        float total = 0.0f;
+        if (mix != nullptr) {
+            float y = 0.0f;
+            for (int p = 0; p < parts; ++p) y += delta[p * part_stride + (size_t)t * width + e];
+#pragma unroll
+            for (int to = 0; to < STREAMS_MAX; ++to) {
+                if (to < R) {
+                    float v = 0.0f;
+#pragma unroll
+                    for (int s = 0; s < STREAMS_MAX; ++s)
+                        if (s < R) v += c.mix[s][to] * x[s];
+                    total += v + c.out[to] * y;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < STREAMS_MAX; ++r)
+                if (r < R) total += x[r];
+        }
+        out[(size_t)i * width + e] = total;
+    }
+}
+
+static int block_for(int width) { return width >= 2048 ? 1024 : (width >= 1024 ? 512 : (width >= 256 ? 256 : 64)); }
+
+extern "C" {
+
+int kipp_streams_open(const void* table, int table_dtype, const int32_t* tokens, float* X, int n, int R, int width,
+                      hipStream_t stream) {
+    if (n <= 0) return 0;
+    if (R <= 0 || R > STREAMS_MAX || width <= 0) return -1;
+    if (table_dtype == KIPP_BF16)
+        hipLaunchKernelGGL(streams_open_kernel<bf16_t>, dim3(n), dim3(block_for(width)), 0, stream, (const bf16_t*)table, tokens, X, R, width);
+    else
+        hipLaunchKernelGGL(streams_open_kernel<float>, dim3(n), dim3(block_for(width)), 0, stream, (const float*)table, tokens, X, R, width);
+    return KIPP_LAUNCH_CHECK();
+}
+
+// delta/mix/outw null: no write.  inw null: no read (h unused).
+int kipp_streams_step(float* X, const float* delta, int parts, const float* mix, const float* outw, const float* inw,
+                      const float* norm_w, float eps, void* h, int h_dtype, int n, int R, int width, hipStream_t stream) {
+    if (n <= 0) return 0;
+    if (R <= 0 || R > STREAMS_MAX || width <= 0 || width > 32768) return -1;
+    if ((mix == nullptr) != (delta == nullptr) || (mix != nullptr && outw == nullptr)) return -2;
+    if (inw != nullptr && (norm_w == nullptr || h == nullptr)) return -2;
+    const size_t lds = (size_t)(width + 16) * sizeof(float);
+    const size_t stride = (size_t)n * width;
+    if (h_dtype == KIPP_BF16)
+        hipLaunchKernelGGL(streams_step_kernel<bf16_t>, dim3(n), dim3(block_for(width)), lds, stream, X, delta, parts, stride, mix, outw,
+                           inw, norm_w, eps, (bf16_t*)h, R, width);
+    else
+        hipLaunchKernelGGL(streams_step_kernel<float>, dim3(n), dim3(block_for(width)), lds, stream, X, delta, parts, stride, mix, outw,
+                           inw, norm_w, eps, (float*)h, R, width);
+    return KIPP_LAUNCH_CHECK();
+}
+
+// `n` tokens in X and delta; `n_out` rows leave (`which` names them, or null: all n in order).
+int kipp_streams_close(const float* X, const float* delta, int parts, const float* mix, const float* outw,
+                       const int32_t* which, float* out, int n, int n_out, int R, int width, hipStream_t stream) {
+    if (n_out <= 0) return 0;
+    if (R <= 0 || R > STREAMS_MAX || width <= 0) return -1;
+    if ((mix == nullptr) != (delta == nullptr) || (mix != nullptr && outw == nullptr)) return -2;
+    hipLaunchKernelGGL(streams_close_kernel, dim3(n_out), dim3(block_for(width)), 0, stream, X, delta, parts, (size_t)n * width, mix,
+                       outw, which, out, R, width);
+    return KIPP_LAUNCH_CHECK();
+}
+
+}  // extern "C"

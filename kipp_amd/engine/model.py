@@ -109,6 +109,8 @@ class Model:
         """Run the batch's tokens through every run of the order; float32 logits
         [wanted, vocab] at `batch.want_rows`, or None if nothing is wanted."""
         batch.step_cache.clear()
+        if self.spec.streams is not None:
+            return self._forward_streams(batch, cache)
         x = self.embedding.forward(batch.tokens)
         if self.input_position is not None:
             x = self.input_position.forward(x, batch)
@@ -132,6 +134,27 @@ class Model:
         rows = ops.gather_rows(x, batch.want_rows, self.rt.empty((batch.n_want, x.shape[1]), torch.float32))
         normed = self.final_norm.forward(rows, self.rt.act_dtype)
         return self.head.forward(normed)
+
+
+def _forward_streams(self, batch, cache) -> Optional[torch.Tensor]:
+    """The forward pass of a model that keeps several copies of the residual stream: x is [tokens, R, width], every
+    copy the token's embedding at the start; the blocks read and write the copies; the final norm reads their sum."""
+    from ..parts.streams import close_streams, open_streams
+    if self.input_position is not None or float(getattr(self.spec.embedding, "scale", 1.0)) != 1.0:
+        raise NotImplementedError("several residual streams with a scaled embedding or a position part on the stream")
+    x = open_streams(self.rt, self.embedding.weight, batch.tokens, self.spec.streams)
+    pending = None
+    for index, run in enumerate(self.spec.order):
+        view = cache.view(index, run.cache_of)
+        x, pending = self.blocks[run.layer].forward(x, pending, batch, view, cache.state(index))
+    if batch.n_want == 0:
+        # nothing is asked for, and the last write has no reader: the step's work for the caches and states is done
+        return None
+    rows = close_streams(self.rt, x, pending, None if batch.want_every_row else batch.want_rows)
+    return self.head.forward(self.final_norm.forward(rows, self.rt.act_dtype))
+
+
+Model._forward_streams = _forward_streams
 
 
 def load_model(model_dir: str, runtime) -> Model:

@@ -15,13 +15,14 @@ from typing import Callable, Dict, Tuple
 class ParamSpec:
     """A tensor a part needs.  kind "float": a matrix or vector of reals;
     "int": an integer table (kept as int32).  `init` is how the random-weights
-    mode fills it: ("normal", std), ("one_plus_normal", std) or ("abs_normal", std)."""
+    mode fills it: ("normal", std), ("one_plus_normal", std), ("abs_normal", std) or ("eye_plus_normal", std)
+    (a square matrix: the identity plus noise)."""
     shape: Tuple[int, ...]
     kind: str = "float"
     init: Tuple[str, float] = ("normal", 0.02)
 
 
-CATEGORIES = ("mixer", "feed_forward", "norm", "position", "block", "embedding", "head")
+CATEGORIES = ("mixer", "feed_forward", "norm", "position", "block", "embedding", "head", "connection")
 _REGISTRY: Dict[str, Dict[str, type]] = {c: {} for c in CATEGORIES}
 
 

@@ -33,8 +33,8 @@ class Embedding:
 
 @register("head", "lm_head")
 class Head:
-    """logits = W x, float32, no bias (/root/reference/src/kipp.c:2660-2661).  A tied
-    head has no tensor of its own and uses the embedding table."""
+    """logits = W x, float32, no bias (/root/reference/src/kipp.c:2660-2661), times the spec's `scale` where
+    that is not 1.  A tied head has no tensor of its own and uses the embedding table."""
 
     graph_safe = True   # forward launches kernels only: no host reads, no data-dependent launches
 
@@ -45,10 +45,12 @@ class Head:
 
     @staticmethod
     def params(spec):
-        return {} if spec.tied else {"weight": ParamSpec((spec.vocab_size, spec.hidden_size))}
+        return {} if spec.tied else {getattr(spec, "name", "weight"): ParamSpec((spec.vocab_size, spec.hidden_size))}
 
     def load(self, tensors, embedding=None):
-        self.weight = self.rt.weight(embedding.weight if self.spec.tied else tensors["weight"])
+        self.weight = self.rt.weight(embedding.weight if self.spec.tied else tensors[getattr(self.spec, "name", "weight")])
 
     def forward(self, x):
-        return self.rt.linear(x, self.weight)
+        logits = self.rt.linear(x, self.weight)
+        scale = float(getattr(self.spec, "scale", 1.0))
+        return logits if scale == 1.0 else self.rt.ops.scale_values(logits, scale)

@@ -43,28 +43,32 @@ class Attention:
 
     @staticmethod
     def params(spec):
-        p = {
-            "q_proj.weight": ParamSpec((spec.q_dim, spec.hidden_size)),
-            "k_proj.weight": ParamSpec((spec.kv_dim, spec.hidden_size)),
-            "v_proj.weight": ParamSpec((spec.kv_dim, spec.hidden_size)),
-            "o_proj.weight": ParamSpec((spec.hidden_size, spec.q_dim)),
-        }
-        if spec.qk_norm_eps is not None:
-            p["q_norm.weight"] = ParamSpec((spec.head_dim,), "float", ("one_plus_normal", 0.05))
-            p["k_norm.weight"] = ParamSpec((spec.head_dim,), "float", ("one_plus_normal", 0.05))
+        q, k, v, o, q_norm, k_norm = spec.names
+        p = {q: ParamSpec((spec.q_dim, spec.hidden_size)), o: ParamSpec((spec.hidden_size, spec.out_dim))}
+        if spec.own_kv:
+            p[k] = ParamSpec((spec.kv_dim, spec.hidden_size))
+            p[v] = ParamSpec((spec.v_dim, spec.hidden_size))
+        if spec.bias:
+            for name, width in zip(spec.bias_names, (spec.q_dim, spec.kv_dim, spec.v_dim)):
+                if spec.own_kv or name == spec.bias_names[0]:
+                    p[name] = ParamSpec((width,), "float", ("normal", 0.1))
+        if spec.qk_norm_eps is not None and spec.qk_norm_weight:
+            p[q_norm] = ParamSpec((spec.head_dim,), "float", ("one_plus_normal", 0.05))
+            p[k_norm] = ParamSpec((spec.head_dim,), "float", ("one_plus_normal", 0.05))
         return p
 
     @staticmethod
     def placement(spec):
-        return {"q_norm.weight": "float32", "k_norm.weight": "float32"}
+        """What enters norms and sums in float32 is widened on the device (exact)."""
+        return {name: "float32" for name in spec.names[4:] + tuple(spec.bias_names)}
 
     @staticmethod
     def variants(spec, dtype):
         """The builds of its specialised kernels (one per head size; decode also per number of query heads
         that share a key/value head).  Under float32, and for more than 16 heads a group, the generic
         attention kernel runs, which every model has."""
-        out = [("rope_kv", None), ("attention_generic", None)]
-        if dtype != "bfloat16" or spec.head_dim % 16:
+        out = [("rope_kv", None) if spec.plain else ("head_prepare", None), ("attention_generic", None)]
+        if dtype != "bfloat16" or spec.head_dim % 16 or spec.value_dim != spec.head_dim:
             return out
         group = spec.num_heads // spec.num_kv_heads
         out.append(("attention_prefill", {"HEAD_DIM": spec.head_dim}))
@@ -74,20 +78,29 @@ class Attention:
 
     def load(self, tensors):
         import torch
-        q, k, v = tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]
-        if not (q.dtype == k.dtype == v.dtype):
-            q, k, v = (t.float() for t in (q, k, v))
+        s = self.spec
+        names = s.names
+        rows = [tensors[names[0]]] + ([tensors[names[1]], tensors[names[2]]] if s.own_kv else [])
+        if len({t.dtype for t in rows}) > 1:
+            rows = [t.float() for t in rows]
         # rows concatenated: one product serves q, k and v; no output element changes
-        self.w_qkv = self.rt.weight(torch.cat([q, k, v], dim=0).contiguous())
-        self.w_o = self.rt.weight(tensors["o_proj.weight"])
-        if self.spec.qk_norm_eps is not None:
-            self.q_norm = tensors["q_norm.weight"]
-            self.k_norm = tensors["k_norm.weight"]
+        self.w_qkv = self.rt.weight(torch.cat(rows, dim=0).contiguous())
+        self.w_o = self.rt.weight(tensors[names[3]])
+        if s.qk_norm_eps is not None and s.qk_norm_weight:
+            self.q_norm = tensors[names[4]]
+            self.k_norm = tensors[names[5]]
+        self.bias = None
+        if s.bias:
+            held = [tensors[name] for name in (s.bias_names if s.own_kv else s.bias_names[:1])]
+            if not s.own_kv:        # the kernel's bias runs over q | k | v: nothing is added where nothing is written
+                held.append(torch.zeros(s.kv_dim + s.v_dim, dtype=torch.float32, device=held[0].device))
+            self.bias = torch.cat([t.float() for t in held]).contiguous()
 
     @staticmethod
     def need_of(spec):
         """What a mixer of this spec keeps per token, known without building it."""
-        return KVNeed(num_kv_heads=spec.num_kv_heads, head_dim=spec.head_dim, window=spec.window, page_size=spec.page_size)
+        return KVNeed(num_kv_heads=spec.num_kv_heads, head_dim=spec.head_dim, window=spec.window, page_size=spec.page_size,
+                      v_head_dim=spec.v_head_dim)
 
     def cache_need(self):
         return self.need_of(self.spec)
@@ -98,6 +111,8 @@ class Attention:
     def forward(self, x, batch, cache, state=None):
         s, rt = self.spec, self.rt
         n = x.shape[0]
+        if not s.plain:
+            return self._forward_prepared(x, batch, cache)
         inv_freq, rotary_dim = self.position.rotary_table()
         angles = self.position.angles(batch) if hasattr(self.position, "angles") and hasattr(batch, "step_cache") else None
         table = batch.block_tables[cache.group]
@@ -124,7 +139,7 @@ class Attention:
             rt.ops.attention_decode_fused(qkv, cache.k, cache.v, out, batch.decode_rows, batch.positions,
                                           batch.seq_of_token, table, s.num_heads, s.num_kv_heads, s.head_dim,
                                           self.q_norm, self.k_norm, eps, inv_freq, rotary_dim, cache.writable,
-                                          self.scale, s.window or 0, batch.max_decode_ctx, self._workspace(batch),
+                                          self.scale, s.window or 0, batch.max_decode_ctx, decode_workspace(rt, batch, s.num_heads, s.head_dim),
                                           angles=angles, out_steps_major=major)
             return rt.linear(out, self.w_o, slabs=True, defer=True, x_steps_major=major)
         q = rt.ops.qk_norm_rope_kv_write(
@@ -132,82 +147,122 @@ class Attention:
             batch.positions, batch.seq_of_token, table, s.num_heads, s.num_kv_heads, s.head_dim,
             self.q_norm, self.k_norm, eps, inv_freq, rotary_dim, write_kv=cache.writable, angles=angles, pairing=pairing)
         out = rt.empty((n, s.q_dim), rt.act_dtype)
-        if fast:
-            if batch.n_portions:
-                item_seq, item_tile, cuts = self._prefill_work(batch)
-                rt.ops.attention_prefill(q, cache.k, cache.v, out, item_seq, item_tile, batch.q_start,
-                                         batch.q_len, batch.positions, table, s.num_heads, s.num_kv_heads, s.head_dim,
-                                         self.scale, s.window or 0, cuts=cuts)
-            if batch.n_decode:
-                rt.ops.attention_decode(q, cache.k, cache.v, out, batch.decode_rows, batch.positions, batch.seq_of_token,
-                                        table, s.num_heads, s.num_kv_heads, s.head_dim, self.scale, s.window or 0,
-                                        batch.max_decode_ctx, self._workspace(batch))
-        else:
-            # the float32 path, and geometries the matrix-core kernels refuse (groups above 16, odd page sizes)
-            rt.ops.paged_attention_generic(q, cache.k, cache.v, out, batch.positions, batch.seq_of_token, table,
-                                           s.num_heads, s.num_kv_heads, s.head_dim, self.scale, s.window or 0)
+        paged_attention(rt, batch, q, out, cache.k, cache.v, cache.page_size, table, s.num_heads, s.num_kv_heads, s.head_dim,
+                        s.head_dim, self.scale, s.window, fast)
         return rt.linear(out, self.w_o, slabs=True, defer=True)
 
-    def _prefill_work(self, batch):
-        """The work list of the prefill kernel: (entry, tile of 128 query rows) for every entry that brings a
-        portion, the longest key range first (the kernel folds the list so that workgroups sharing a
-        compute unit carry about the same load).
+    def _forward_prepared(self, x, batch, cache):
+        """The mixer without rotation and with any of: biases, a norm without weights, a factor on the queries that grows
+        with the position, values of their own width, keys and values of another run.  One kernel makes the heads ready
+        from the input product; the attention kernels are the same."""
+        s, rt = self.spec, self.rt
+        if self.position.rotary_table()[0] is not None:
+            raise NotImplementedError("an attention mixer with biases, a plain norm, a query factor or its own value width does not rotate")
+        n = x.shape[0]
+        table = batch.block_tables[cache.group]
+        d, dv = s.head_dim, s.value_dim
+        if not s.own_kv and cache.writable:
+            raise ValueError("an attention mixer without key and value projections needs the cache of another run")
+        proj = rt.linear(rt.rows_of(x), self.w_qkv, slabs=True)
+        norm = "none" if s.qk_norm_eps is None else ("weighted" if s.qk_norm_weight else "plain")
+        coef, every = s.q_temp if s.q_temp is not None else (0.0, 0)
+        # (without projections of its own only q was projected: its columns stand at the row's start all the same)
+        q = rt.ops.head_prepare(proj, rt.empty((n, s.q_dim), rt.act_dtype), cache.k, cache.v, batch.positions,
+                                batch.seq_of_token, table, s.num_heads, s.num_kv_heads, d, dv, self.bias, norm,
+                                s.qk_norm_eps or 0.0, self.q_norm, self.k_norm, coef, every,
+                                write_kv=cache.writable and s.own_kv)
+        fast = rt.dtype == "bfloat16" and d % 16 == 0 and d == dv \
+            and rt.ops.attention_fast_ok(s.num_heads, s.num_kv_heads, cache.page_size, table.shape[1])
+        if rt.dtype == "bfloat16" and not fast:
+            rt.generic_attention_launches += 1
+        out = rt.empty((n, s.out_dim), rt.act_dtype)
+        paged_attention(rt, batch, q, out, cache.k, cache.v, cache.page_size, table, s.num_heads, s.num_kv_heads, d, dv,
+                        self.scale, s.window, fast)
+        return rt.linear(out, self.w_o, slabs=True, defer=True)
 
-        A workgroup walks all keys its tile sees, one after the other.  Where the tiles times the heads are
-        fewer workgroups than two a compute unit and the contexts are long (a portion of a few hundred rows
-        behind thousands of keys), the keys are cut as well, at multiples of a length chosen so that the
-        GPU is filled about twice: a work item is then (entry, tile, cut), and the cuts of a row are merged
-        in order afterwards.  The cuts follow from the step's shape, not from a row's place in it, so a row's
-        result may differ in its last bits between steps of different shapes, as between the kernels for
-        portions and for single tokens.  Made by the first attention layer of a forward pass and shared by
-        the others of the same geometry."""
-        s, ops = self.spec, self.rt.ops
-        key = ("attention_prefill_work", s.num_heads, s.head_dim, s.window)
-        work = batch.step_cache.get(key)
-        if work is None:
-            tile = ops.PREFILL_ROWS
-            q_start = batch.host["q_start"]
-            portions = [(i, n, ctx) for i, (n, ctx) in enumerate(zip(batch.host["q_len"], batch.host["ctx_len"])) if n > 1]
-            tiles = [(i, t, ctx - n + min((t + 1) * tile, n) - 1, q_start[i] + t * tile, min(tile, n - t * tile))
-                     for i, n, ctx in portions for t in range((n + tile - 1) // tile)]     # (entry, tile, last key, first row, rows)
-            workgroups = len(tiles) * s.num_heads
-            longest = max(last for _, _, last, _, _ in tiles) + 1
-            split_keys = 0
-            units = ops.compute_units(self.rt.device)
-            if s.window is None and workgroups < 2 * units:
-                want = -(-2 * units // workgroups)
-                split_keys = max(ops.PREFILL_MIN_CUT, -(-longest // want // 64) * 64)
-                if longest <= split_keys:
-                    split_keys = 0
-            if not split_keys:
-                items = sorted((-last, i, t) for i, t, last, _, _ in tiles)
-                work = tuple(batch.upload([i for _, i, _ in items], [t for _, _, t in items])) + (None,)
-            else:
-                items, merge_rows, merge_cuts = [], [], []
-                for i, t, last, row0, rows in tiles:
-                    cuts = last // split_keys + 1
-                    items.extend((-(min(last + 1, (c + 1) * split_keys) - c * split_keys), i, t, c) for c in range(cuts))
-                    merge_rows.extend(range(row0, row0 + rows))
-                    merge_cuts.extend([cuts] * rows)
-                items.sort()
-                most = max(merge_cuts)
-                seq, til, cut, rows_d, cuts_d = batch.upload([i for _, i, _, _ in items], [t for _, _, t, _ in items],
-                                                             [c for _, _, _, c in items], merge_rows, merge_cuts)
-                space = ops.attention_prefill_workspace(batch.n_tokens, s.num_heads, s.head_dim, most, self.rt.device)
-                work = (seq, til, (split_keys, cut, rows_d, cuts_d, space))
-            batch.step_cache[key] = work
-        return work
 
-    def _workspace(self, batch):
-        """Partial results of the split decode kernel, shared by the layers of one geometry and kept
-        while the batch object lives (a recorded step keeps its own)."""
-        s = self.spec
-        key = ("decode_workspace", batch.n_decode, batch.max_decode_ctx, s.num_heads, s.head_dim)
-        ws = batch.host.get(key)
-        if ws is None:
-            ws = self.rt.ops.attention_decode_workspace(batch.n_decode, s.num_heads, s.head_dim,
-                                                        batch.max_decode_ctx, self.rt.device)
-            if not self.rt.merge_in_kernel:
-                ws = ws[:2]         # without the counts the splits are merged by a launch of its own
-            batch.host[key] = ws
-        return ws
+def paged_attention(rt, batch, q, out, k_cache, v_cache, page_size, table, n_q, n_kv, d, dv, scale, window, fast):
+    """The attention itself over a paged cache, for any mixer that has its queries ready: q [tokens, n_q d] -> out
+    [tokens, n_q dv].  `fast`: the matrix-core kernels (prompt portions and single tokens each by their own; they
+    need d == dv, or `v_cache` being `k_cache`, a value then being as wide as its key's row); else the generic kernel,
+    which takes values of their own width (`v_cache` may be `k_cache` there too: a value is the first dv numbers
+    of its key's row)."""
+    if fast:
+        if batch.n_portions:
+            item_seq, item_tile, cuts = prefill_work(rt, batch, n_q, d, window)
+            rt.ops.attention_prefill(q, k_cache, v_cache, out, item_seq, item_tile, batch.q_start, batch.q_len, batch.positions,
+                                     table, n_q, n_kv, d, scale, window or 0, cuts=cuts)
+        if batch.n_decode:
+            rt.ops.attention_decode(q, k_cache, v_cache, out, batch.decode_rows, batch.positions, batch.seq_of_token, table,
+                                    n_q, n_kv, d, scale, window or 0, batch.max_decode_ctx, decode_workspace(rt, batch, n_q, d))
+    elif d == dv and v_cache is not k_cache and d <= 256:
+        # the float32 path, and geometries the matrix-core kernels refuse (groups above 16, odd page sizes)
+        rt.ops.paged_attention_generic(q, k_cache, v_cache, out, batch.positions, batch.seq_of_token, table, n_q, n_kv, d,
+                                       scale, window or 0)
+    else:
+        rt.ops.paged_attention_wide(q, k_cache, v_cache, out, batch.positions, batch.seq_of_token, table, n_q, n_kv, d, dv,
+                                    scale, window or 0)
+    return out
+
+
+def prefill_work(rt, batch, num_heads, head_dim, window):
+    """The work list of the prefill kernel: (entry, tile of 128 query rows) for every entry that brings a
+    portion, the longest key range first (the kernel folds the list so that workgroups sharing a
+    compute unit carry about the same load).
+
+    A workgroup walks all keys its tile sees, one after the other.  Where the tiles times the heads are
+    fewer workgroups than two a compute unit and the contexts are long (a portion of a few hundred rows
+    behind thousands of keys), the keys are cut as well, at multiples of a length chosen so that the
+    GPU is filled about twice: a work item is then (entry, tile, cut), and the cuts of a row are merged
+    in order afterwards.  The cuts follow from the step's shape, not from a row's place in it, so a row's
+    result may differ in its last bits between steps of different shapes, as between the kernels for
+    portions and for single tokens.  Made by the first attention layer of a forward pass and shared by
+    the others of the same geometry."""
+    ops = rt.ops
+    key = ("attention_prefill_work", num_heads, head_dim, window)
+    work = batch.step_cache.get(key)
+    if work is None:
+        tile = ops.PREFILL_ROWS
+        q_start = batch.host["q_start"]
+        portions = [(i, n, ctx) for i, (n, ctx) in enumerate(zip(batch.host["q_len"], batch.host["ctx_len"])) if n > 1]
+        tiles = [(i, t, ctx - n + min((t + 1) * tile, n) - 1, q_start[i] + t * tile, min(tile, n - t * tile))
+                 for i, n, ctx in portions for t in range((n + tile - 1) // tile)]     # (entry, tile, last key, first row, rows)
+        workgroups = len(tiles) * num_heads
+        longest = max(last for _, _, last, _, _ in tiles) + 1
+        split_keys = 0
+        units = ops.compute_units(rt.device)
+        if window is None and workgroups < 2 * units:
+            want = -(-2 * units // workgroups)
+            split_keys = max(ops.PREFILL_MIN_CUT, -(-longest // want // 64) * 64)
+            if longest <= split_keys:
+                split_keys = 0
+        if not split_keys:
+            items = sorted((-last, i, t) for i, t, last, _, _ in tiles)
+            work = tuple(batch.upload([i for _, i, _ in items], [t for _, _, t in items])) + (None,)
+        else:
+            items, merge_rows, merge_cuts = [], [], []
+            for i, t, last, row0, rows in tiles:
+                cuts = last // split_keys + 1
+                items.extend((-(min(last + 1, (c + 1) * split_keys) - c * split_keys), i, t, c) for c in range(cuts))
+                merge_rows.extend(range(row0, row0 + rows))
+                merge_cuts.extend([cuts] * rows)
+            items.sort()
+            most = max(merge_cuts)
+            seq, til, cut, rows_d, cuts_d = batch.upload([i for _, i, _, _ in items], [t for _, _, t, _ in items],
+                                                         [c for _, _, _, c in items], merge_rows, merge_cuts)
+            space = ops.attention_prefill_workspace(batch.n_tokens, num_heads, head_dim, most, rt.device)
+            work = (seq, til, (split_keys, cut, rows_d, cuts_d, space))
+        batch.step_cache[key] = work
+    return work
+
+def decode_workspace(rt, batch, num_heads, head_dim):
+    """Partial results of the split decode kernel, shared by the layers of one geometry and kept
+    while the batch object lives (a recorded step keeps its own)."""
+    key = ("decode_workspace", batch.n_decode, batch.max_decode_ctx, num_heads, head_dim)
+    ws = batch.host.get(key)
+    if ws is None:
+        ws = rt.ops.attention_decode_workspace(batch.n_decode, num_heads, head_dim, batch.max_decode_ctx, rt.device)
+        if not rt.merge_in_kernel:
+            ws = ws[:2]         # without the counts the splits are merged by a launch of its own
+        batch.host[key] = ws
+    return ws

@@ -34,15 +34,15 @@ class RMSNorm:
 
     @staticmethod
     def params(spec):
-        return {"weight": ParamSpec((spec.width,), "float", ("one_plus_normal", 0.05))}
+        return {getattr(spec, "name", "weight"): ParamSpec((spec.width,), "float", ("one_plus_normal", 0.05))}
 
     @staticmethod
     def placement(spec):
         """Norm weights are widened to float32 on the device (exact)."""
-        return {"weight": "float32"}
+        return {getattr(spec, "name", "weight"): "float32"}
 
     def load(self, tensors):
-        self.weight = tensors["weight"]
+        self.weight = tensors[getattr(self.spec, "name", "weight")]
 
     def forward(self, x, out_dtype):
         return self.rt.ops.rmsnorm(x, self.weight, self.spec.eps, self.rt.empty(x.shape, out_dtype))

@@ -90,3 +90,29 @@ class Rope:
                                               self.rt.empty((batch.n_tokens, self.rotary_dim), torch.float32))
             batch.step_cache[key] = table
         return table
+
+
+@register("position", "rope_scaled")
+class ScaledRope(Rope):
+    """Rotary frequencies stretched for contexts beyond the length a model was made for (`ScaledRopeSpec` has the
+    rule): dimensions that turn often over that length keep their frequency, those that turn rarely are slowed by
+    `factor`, a ramp blends between them, and cosines and sines are multiplied by `magnitude` = 0.1 ln(factor) + 1.
+    The table is computed once in float64 and rounded to float32; the angle product is float32."""
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        import math
+        self.magnitude = 0.1 * math.log(float(spec.factor)) + 1.0
+
+    def frequencies(self) -> torch.Tensor:
+        import math
+        s, dims = self.spec, self.rotary_dim
+        plain = super().frequencies()
+
+        def turn_dim(turns: float) -> float:
+            return dims * math.log(float(s.original) / (2.0 * math.pi * turns)) / (2.0 * math.log(float(s.theta)))
+        lo = max(math.floor(turn_dim(float(s.fast))), 0)
+        hi = min(math.ceil(turn_dim(float(s.slow))), dims - 1)
+        i = torch.arange(dims // 2, dtype=torch.float64)
+        ramp = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        return plain / float(s.factor) * ramp + plain * (1.0 - ramp)

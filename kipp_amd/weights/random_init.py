@@ -39,6 +39,8 @@ def random_tensor(seed: int, name: str, spec: ParamSpec, dtype: torch.dtype = to
         t += 1.0
     elif how == "abs_normal":
         t.abs_()
+    elif how == "eye_plus_normal":
+        t += torch.eye(spec.shape[0], spec.shape[1], dtype=torch.float32, device=device)
     elif how != "normal":
         raise ValueError(f"unknown init {how!r} for {name}")
     return t.to(dtype)
