@@ -253,8 +253,8 @@ class MLSTMSpec:
     names: Tuple[str, ...] = ("q", "k", "v", "g", "o", "norm", "i", "i.b", "f", "f.b")
 
     def __post_init__(self):
-        if self.num_heads <= 0 or self.v_head_dim <= 0 or not 0 < self.head_dim <= 256:
-            raise ConfigError("mlstm: heads and value size must be positive, key size from 1 to 256")
+        if self.num_heads <= 0 or self.v_head_dim <= 0 or not 0 < self.head_dim <= 1024:
+            raise ConfigError("mlstm: heads and value size must be positive, key size from 1 to 1,024")
         if not self.gate_cap > 0:
             raise ConfigError(f"mlstm: gate_cap must be positive, got {self.gate_cap}")
         if len(self.names) != 10:

@@ -8,7 +8,7 @@
 //     m' = max(lf + m, li)
 //     S' = exp(lf + m - m') S + exp(li - m') k v^T       (d x dv),   n' likewise with k alone
 //     o  = S'^T q / (max(|n' . q|, exp(-m')) + 1e-6)
-// S, n and m live in the request's state slot as float32 [heads][d][dv] | [Z][heads][d] | [Z][heads], Z = ceil(dv / 64):
+// S, n and m live in the request's state slot as float32 [heads][d][dv] | [Z][heads][d] | [Z][heads], Z = ceil(dv / columns of a workgroup):
 // every workgroup of a head keeps a copy of n and m of its own (all equal), so that none reads what another has
 // already written for the next step.  A slot that was just claimed holds zeros, which is the recurrence's start.
 // Everything here is float32.
@@ -16,7 +16,7 @@
 // scan    a workgroup takes (entry of the batch, head, 64 columns of S) and walks the entry's tokens in order.
 //         A column is shared by 4 lanes that stand side by side in a wave, each with every fourth row of it, so
 //         the sum over rows ends in two lane exchanges and no wave waits for another: there is no barrier in
-//         the walk.  Every lane also keeps its rows of n (the same arithmetic in every column, hence the same
+//         the walk.  (Keys of more than 256 numbers: 16 lanes a column, 16 columns a workgroup.)  Every lane also keeps its rows of n (the same arithmetic in every column, hence the same
 //         bits), so the denominator needs no exchange between columns either.
 // finish  every head of a token divided by its root mean square, times the norm's weight, times sigmoid(gate),
 //         in the type the output projection reads.
@@ -26,16 +26,16 @@
 #include "common.h"
 #include <math.h>
 
-#define SCAN_PARTS 4
-#define SCAN_COLS 64
+#define SCAN_THREADS 256
 
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.0f) - log1pf(expf(-fabsf(z))); }
 
-template <int ROWS>     // rows of a column that one lane holds: ceil(d / SCAN_PARTS) <= ROWS
-__global__ void __launch_bounds__(SCAN_PARTS * SCAN_COLS) mlstm_scan_kernel(
+template <int ROWS, int SCAN_PARTS>     // rows of a column that one lane holds: ceil(d / SCAN_PARTS) <= ROWS
+__global__ void __launch_bounds__(SCAN_THREADS) mlstm_scan_kernel(
     const float* __restrict__ proj, int stride, const float* __restrict__ bias_i, const float* __restrict__ bias_f, float cap,
     float* __restrict__ state, size_t state_stride, const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
     const int32_t* __restrict__ slots, float* __restrict__ o_raw, int heads, int d, int dv) {
+    constexpr int SCAN_COLS = SCAN_THREADS / SCAN_PARTS;
     const int seq = blockIdx.x, head = blockIdx.y;
     const int part = threadIdx.x & (SCAN_PARTS - 1);
     const int col = blockIdx.z * SCAN_COLS + threadIdx.x / SCAN_PARTS;
@@ -77,10 +77,11 @@ __global__ void __launch_bounds__(SCAN_PARTS * SCAN_COLS) mlstm_scan_kernel(
             num = fmaf(S[r], q, num);
             den = fmaf(nv[r], q, den);
         }
-        num += __shfl_xor(num, 1, KIPP_WAVE);
-        num += __shfl_xor(num, 2, KIPP_WAVE);
-        den += __shfl_xor(den, 1, KIPP_WAVE);
-        den += __shfl_xor(den, 2, KIPP_WAVE);
+#pragma unroll
+        for (int off = 1; off < SCAN_PARTS; off <<= 1) {
+            num += __shfl_xor(num, off, KIPP_WAVE);
+            den += __shfl_xor(den, off, KIPP_WAVE);
+        }
         m = m_new;
         if (live && part == 0)
             o_raw[((size_t)t * heads + head) * dv + col] = num / (fmaxf(fabsf(den), expf(-m)) + 1e-6f);
@@ -119,18 +120,21 @@ int kipp_mlstm_scan(const float* proj, int stride, const float* bias_i, const fl
                     size_t state_stride, const int32_t* q_start, const int32_t* q_len, const int32_t* slots, float* o_raw,
                     int n_seqs, int heads, int d, int dv, hipStream_t stream) {
     if (n_seqs <= 0) return 0;
-    if (heads <= 0 || d <= 0 || d > 256 || dv <= 0 || !(cap > 0.0f)) return -1;
-    if (stride < 2 * heads * d + 2 * heads * dv + 2 * heads || state_stride < (size_t)heads * d * dv + (size_t)((dv + SCAN_COLS - 1) / SCAN_COLS) * (heads * d + heads)) return -1;
-    dim3 grid(n_seqs, heads, (dv + SCAN_COLS - 1) / SCAN_COLS), block(SCAN_PARTS * SCAN_COLS);
-    const int rows = (d + SCAN_PARTS - 1) / SCAN_PARTS;
-#define KIPP_SCAN(R)                                                                                                        \
-    hipLaunchKernelGGL(mlstm_scan_kernel<R>, grid, block, 0, stream, proj, stride, bias_i, bias_f, cap, state, state_stride, \
+    if (heads <= 0 || d <= 0 || d > 1024 || dv <= 0 || !(cap > 0.0f)) return -1;
+    const int parts = d <= 256 ? 4 : 16;
+    const int cols = SCAN_THREADS / parts;
+    if (stride < 2 * heads * d + 2 * heads * dv + 2 * heads || state_stride < (size_t)heads * d * dv + (size_t)((dv + cols - 1) / cols) * (heads * d + heads)) return -1;
+    dim3 grid(n_seqs, heads, (dv + cols - 1) / cols), block(SCAN_THREADS);
+    const int rows = (d + parts - 1) / parts;
+#define KIPP_SCAN(R, P)                                                                                                        \
+    hipLaunchKernelGGL((mlstm_scan_kernel<R, P>), grid, block, 0, stream, proj, stride, bias_i, bias_f, cap, state, state_stride, \
                        q_start, q_len, slots, o_raw, heads, d, dv)
-    if (rows <= 4) KIPP_SCAN(4);
-    else if (rows <= 8) KIPP_SCAN(8);
-    else if (rows <= 16) KIPP_SCAN(16);
-    else if (rows <= 32) KIPP_SCAN(32);
-    else KIPP_SCAN(64);
+    if (parts == 16) KIPP_SCAN(64, 16);
+    else if (rows <= 4) KIPP_SCAN(4, 4);
+    else if (rows <= 8) KIPP_SCAN(8, 4);
+    else if (rows <= 16) KIPP_SCAN(16, 4);
+    else if (rows <= 32) KIPP_SCAN(32, 4);
+    else KIPP_SCAN(64, 4);
 #undef KIPP_SCAN
     return KIPP_LAUNCH_CHECK();
 }

@@ -521,13 +521,15 @@ def latent_expand(lat: torch.Tensor, w_uv_t: torch.Tensor, out: torch.Tensor, he
 
 # --------------------------------------------------------------------------- matrix memory (mLSTM)
 
-MLSTM_COLS = 64     # columns of the memory a workgroup of the scan takes
+def mlstm_columns(d: int) -> int:
+    """Columns of the memory that a workgroup of the scan takes (fewer where a column's rows need more lanes)."""
+    return 64 if d <= 256 else 16
 
 
 def mlstm_state_size(heads: int, d: int, dv: int) -> int:
     """float32 numbers of a request's state: S [heads, d, dv], then a copy of n [heads, d] and m [heads] for every
-    MLSTM_COLS columns."""
-    return heads * d * dv + -(-dv // MLSTM_COLS) * (heads * d + heads)
+    workgroup's columns."""
+    return heads * d * dv + -(-dv // mlstm_columns(d)) * (heads * d + heads)
 
 
 def mlstm_scan(proj: torch.Tensor, bias_i: torch.Tensor, bias_f: torch.Tensor, cap: float, state: torch.Tensor,
@@ -544,8 +546,8 @@ def mlstm_scan(proj: torch.Tensor, bias_i: torch.Tensor, bias_f: torch.Tensor, c
     _need(state.dim() == 2 and state.dtype == torch.float32 and state.shape[1] >= mlstm_state_size(heads, d, dv),
           "mlstm_scan: state is float32 [slots, size]")
     _need(bias_i.dtype == bias_f.dtype == torch.float32 and bias_i.numel() == heads and bias_f.numel() == heads, "mlstm_scan: float32 gate biases [heads]")
-    _need(o_raw.dtype == torch.float32 and o_raw.shape == (proj.shape[0], heads * dv) and 0 < d <= 256 and cap > 0,
-          "mlstm_scan: o_raw is float32 [tokens, heads dv]; key size up to 256")
+    _need(o_raw.dtype == torch.float32 and o_raw.shape == (proj.shape[0], heads * dv) and 0 < d <= 1024 and cap > 0,
+          "mlstm_scan: o_raw is float32 [tokens, heads dv]; key size up to 1,024")
     _need(q_start.numel() == q_len.numel() == slots.numel(), "mlstm_scan: one start, length and slot an entry")
     fn = _fn("mlstm", "kipp_mlstm_scan", [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_size, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                           _c_int, _c_int, _c_int, _c_int, _c_ptr])
