@@ -62,7 +62,7 @@ def prebuilt() -> List[Spec]:
 # alone and in small models, and builds of the decode attention whose thresholds are lowered so that a check can
 # reach the kernels for long contexts and many sequences with inputs it can verify.  `build()` compiles them ahead
 # together with `prebuilt()`; whoever finds one missing compiles it then.
-ATTENTION = [(128, 16), (128, 1), (16, 3), (48, 3), (64, 1), (32, 16), (256, 4), (80, 3), (256, 2), (16, 1), (32, 2), (16, 6)]   # (head size, group)
+ATTENTION = [(128, 16), (128, 1), (16, 3), (48, 3), (64, 1), (32, 16), (256, 4), (80, 3), (256, 2), (16, 1), (32, 2), (16, 6), (64, 4), (256, 16)]   # (head size, group)
 EARLY_STREAM = [(128, 4), (48, 3), (16, 2)]      # the kernel for long contexts takes over at 1,024 keys
 WHOLE_CONTEXTS = [(128, 4), (128, 16)]           # the whole-context kernel at few sequences
 MIXED_HEADS = [(6, 3, 32, 16), (4, 4, 32, 32), (8, 2, 64, 48), (12, 4, 32, 64), (2, 1, 96, 16), (32, 8, 32, 16), (4, 2, 32, 16), (32, 8, 128, 128), (16, 4, 32, 16)]   # (heads, key/value heads, key size, value size) of the attention with mixed heads
