@@ -257,6 +257,35 @@ def tobinex_config(qwen: dict, layers: int, window) -> dict:
                        for _ in range(layers)]}
 
 
+def rerizen_config(qwen: dict, layers: int, kind: str) -> dict:
+    """A Rerizen configuration with the layer sizes of a Qwen3 shape (width, feed-forward, vocabulary, and for the
+    attention mixer the same heads and head size), two residual streams, and `layers` layers of one mixer, so that every
+    mixer's kernels stand beside Qwen3's alone: "attention" (biases, plain head norm, query factor; every second layer
+    reads the keys and values of the one before), "latent" (16 heads over a cached row of 192 + 64 numbers, a window of
+    1,024 keys: the sizes the matrix-core attention takes), "latent_wide" (a cached row of 512 + 64 numbers, which only
+    the generic attention kernel takes), "mlstm" (8 heads whose values fill the width), or "mixed" (one of each in turn)."""
+    width, heads = qwen["hidden_size"], qwen["num_attention_heads"]
+    head_dim = qwen.get("head_dim") or width // heads
+    attention = {"heads": heads, "kv_heads": qwen["num_key_value_heads"], "dim": head_dim, "vdim": head_dim, "scale": head_dim ** -0.5,
+                 "q_temp": {"coef": 0.1, "every": 512}}
+    rot = {"base": 10000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}
+    latent = {"heads": 16, "dim": 128, "rot_dim": 64, "vdim": 128, "q_rank": 768, "kv_rank": 192, "scale": 192 ** -0.5, "rot": rot,
+              "mask": {"size": 1024}}
+    mlstm = {"heads": 8, "dim": 128 if width <= 2560 else 256, "vdim": width // 8, "gate_cap": 15.0}
+    mixers = {"attention": ("attention", attention), "latent": ("latent_attention", latent),
+              "latent_wide": ("latent_attention", dict(latent, kv_rank=512, scale=192 ** -0.5)), "mlstm": ("mlstm", mlstm)}
+    order = ["latent", "attention", "attention", "mlstm"] if kind == "mixed" else [kind]
+    made = []
+    for i in range(layers):
+        name, mixer = mixers[order[i % len(order)]]
+        mixer = dict(mixer)
+        if name == "attention" and i % 2 == 1 and made[-1]["type"] == "attention" and "kv_from" not in made[-1]["mixer"]:
+            mixer["kv_from"] = i - 1
+        made.append({"type": name, "mixer": mixer, "mlp": {"kind": "dense", "ff": qwen["intermediate_size"]}})
+    return {"architecture": "Rerizen", "vocab": qwen["vocab_size"], "width": width, "streams": 2, "logit_scale": 1.0,
+            "norm": {"eps": 1e-6}, "max_position": 8192, "layers": made}
+
+
 def design_points(config, args, label):
     """Prefill of one 2,048-token prompt and decode steps at two batch sizes behind such prompts, for one model made
     with random weights: milliseconds, tokens a second, and what the kernels ran as (recorded steps, library products,
@@ -305,6 +334,24 @@ def design_points(config, args, label):
     return out
 
 
+def rerizen_bench(args) -> int:
+    """`--design rerizen`: the Rerizen design beside Qwen3 at equal layer sizes, a few layers of each, random weights: one
+    model for each of its mixers alone, and one with all of them in turn."""
+    from kipp_amd.config import shape_config
+    layers = args.layers or 4
+    sizes = {}
+    for shape in [s for s in args.design_shapes.split(",") if s]:
+        qwen = shape_config(shape)
+        qwen["num_hidden_layers"] = layers
+        sizes[shape] = {"qwen3": design_points(qwen, args, f"{shape} qwen3")}
+        for kind in [k for k in args.design_kinds.split(",") if k]:
+            sizes[shape][f"rerizen_{kind}"] = design_points(rerizen_config(qwen, layers, kind), args, f"{shape} rerizen, {kind}")
+    print(json.dumps({"metric": "prefill and decode of the Rerizen design beside Qwen3 at equal layer sizes (bf16, random weights)",
+                      "design": "rerizen", "layers": layers, "prompt_tokens": args.prompt, "steps": args.steps,
+                      "unit": "ms and tok/s", "n_gpus": 1, "dtype": "bf16", "data": "synthetic", "sizes": sizes}), flush=True)
+    return 0
+
+
 def design_bench(args) -> int:
     """`--design tobinex`: the Tobinex design beside Qwen3 at equal layer sizes (both with every key kept, and Tobinex
     once more with a window of 1,024 keys behind 4 kept ones), a few layers of each, random weights."""
@@ -344,13 +391,17 @@ def main():
     ap.add_argument("--no-c-host", action="store_true", help="leave out the points measured through the C host")
     ap.add_argument("--products", choices=["default", "own", "auto", "library"], default="default",
                     help="products of many rows (prompt portions): the runtime's default, our kernel only, the fastest of ours and the library's, the library's")
-    ap.add_argument("--design", choices=["tobinex"], default=None,
+    ap.add_argument("--design", choices=["tobinex", "rerizen"], default=None,
                     help="instead of the default workload: this design beside Qwen3 at equal layer sizes (prefill and decode, a few layers)")
     ap.add_argument("--design-shapes", default="qwen3-4b,qwen3-8b", help="the Qwen3 shapes whose layer sizes --design takes")
+    ap.add_argument("--design-kinds", default="attention,latent,latent_wide,mlstm,mixed",
+                    help="--design rerizen: the models that are measured, one mixer each or all in turn")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.design == "rerizen":
+        return rerizen_bench(args)
     if args.design:
         return design_bench(args)
 

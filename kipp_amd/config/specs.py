@@ -219,8 +219,8 @@ class LatentAttentionSpec:
                 raise ConfigError(f"latent attention: {what} must be positive, got {v}")
         if self.rot_dim < 0:
             raise ConfigError(f"latent attention: rot_dim must not be negative, got {self.rot_dim}")
-        if self.kv_rank + self.rot_dim > 1024 or self.head_dim > 2048 or self.kv_rank > 2048:
-            raise ConfigError("latent attention: the cached row (kv_rank + rot_dim) takes up to 1,024 numbers, head_dim and kv_rank up to 2,048")
+        if self.kv_rank + self.rot_dim > 1024 or self.head_dim > 1024:
+            raise ConfigError("latent attention: the cached row (kv_rank + rot_dim) and head_dim take up to 1,024 numbers")
         if self.window is not None and self.window <= 0:
             raise ConfigError(f"attention window must be positive, got {self.window}")
         if len(self.names) != 9:

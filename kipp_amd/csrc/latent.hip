@@ -86,21 +86,67 @@ __global__ void latent_prepare_kernel(
     }
 }
 
-#define ABSORB_TOKENS 8
+#define TILE_TOKENS 8       // tokens of a workgroup of absorb and of expand: a weight is read once for all of them
+#define TILE_COLS 64        // output columns of a workgroup (a lane a column, so that a wave reads a run of a weight row)
+#define TILE_WAVES 4        // the contraction is shared out over the waves and summed through LDS
 
-// One workgroup a (tile of ABSORB_TOKENS tokens, head): a weight row is read once for the tile.
-// LDS: ABSORB_TOKENS * d floats.
+// acc[r] += sum over this wave's share of e of in_s[r][e] * w[e][c]: four weight rows asked for at a time.
+template <typename TW>
+__device__ __forceinline__ void tile_product(const float* in_s, int k, const TW* w, int n, int c, bool live, float (&acc)[TILE_TOKENS]) {
+    const int wave = threadIdx.x / KIPP_WAVE;
+    const int share = (k + TILE_WAVES - 1) / TILE_WAVES;
+    const int e0 = wave * share, e1 = min(k, e0 + share);
+#pragma unroll
+    for (int r = 0; r < TILE_TOKENS; ++r) acc[r] = 0.0f;
+    if (!live) return;
+    int e = e0;
+    for (; e + 4 <= e1; e += 4) {
+        float wv[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) wv[u] = load_f(w, (size_t)(e + u) * n + c);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int r = 0; r < TILE_TOKENS; ++r) acc[r] = fmaf(in_s[r * k + e + u], wv[u], acc[r]);
+    }
+    for (; e < e1; ++e) {
+        const float wv = load_f(w, (size_t)e * n + c);
+#pragma unroll
+        for (int r = 0; r < TILE_TOKENS; ++r) acc[r] = fmaf(in_s[r * k + e], wv, acc[r]);
+    }
+}
+
+// The waves' partial sums added in wave order; every thread of wave 0 gets its column's totals.  red: TILE_WAVES * TILE_TOKENS * TILE_COLS floats.
+__device__ __forceinline__ void tile_reduce(float* red, float (&acc)[TILE_TOKENS]) {
+    const int wave = threadIdx.x / KIPP_WAVE, lane = threadIdx.x & (KIPP_WAVE - 1);
+#pragma unroll
+    for (int r = 0; r < TILE_TOKENS; ++r) red[(wave * TILE_TOKENS + r) * TILE_COLS + lane] = acc[r];
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+        for (int r = 0; r < TILE_TOKENS; ++r) {
+            float total = 0.0f;
+#pragma unroll
+            for (int w = 0; w < TILE_WAVES; ++w) total += red[(w * TILE_TOKENS + r) * TILE_COLS + lane];
+            acc[r] = total;
+        }
+    }
+}
+
+// One workgroup a (tile of tokens, head, 64 columns of the latent).  LDS: TILE_TOKENS * d floats, then the partial sums.
 template <typename TW, typename TO>
-__global__ void latent_absorb_kernel(
+__global__ void __launch_bounds__(TILE_WAVES * KIPP_WAVE) latent_absorb_kernel(
     const float* __restrict__ q, int parts, size_t part_stride, const TW* __restrict__ w_uk, TO* __restrict__ out,
     const int32_t* __restrict__ positions, const float* __restrict__ freq, int rot_dims, float magnitude,
     int n_tokens, int heads, int d, int dr, int rank) {
-    extern __shared__ float q_s[];
-    const int t0 = blockIdx.x * ABSORB_TOKENS;
+    extern __shared__ float lds[];
+    float* q_s = lds;
+    float* red = lds + TILE_TOKENS * d;
+    const int t0 = blockIdx.x * TILE_TOKENS;
     const int head = blockIdx.y;
-    const int rows = min(ABSORB_TOKENS, n_tokens - t0);
+    const int rows = min(TILE_TOKENS, n_tokens - t0);
     const int q_row = heads * (d + dr);
-    for (int i = threadIdx.x; i < ABSORB_TOKENS * d; i += blockDim.x) {
+    for (int i = threadIdx.x; i < TILE_TOKENS * d; i += blockDim.x) {
         const int r = i / d, e = i - r * d;
         float v = 0.0f;
         if (r < rows)
@@ -108,23 +154,19 @@ __global__ void latent_absorb_kernel(
         q_s[i] = v;
     }
     __syncthreads();
-    const TW* w = w_uk + (size_t)head * d * rank;
     const int width = rank + dr;
-    for (int c = threadIdx.x; c < rank; c += blockDim.x) {
-        float acc[ABSORB_TOKENS];
+    const int c = blockIdx.z * TILE_COLS + (threadIdx.x & (KIPP_WAVE - 1));
+    float acc[TILE_TOKENS];
+    tile_product(q_s, d, w_uk + (size_t)head * d * rank, rank, c, c < rank, acc);
+    tile_reduce(red, acc);
+    if (threadIdx.x < KIPP_WAVE && c < rank) {
 #pragma unroll
-        for (int r = 0; r < ABSORB_TOKENS; ++r) acc[r] = 0.0f;
-        for (int e = 0; e < d; ++e) {
-            const float wv = load_f(w, (size_t)e * rank + c);
-#pragma unroll
-            for (int r = 0; r < ABSORB_TOKENS; ++r) acc[r] = fmaf(q_s[r * d + e], wv, acc[r]);
-        }
-#pragma unroll
-        for (int r = 0; r < ABSORB_TOKENS; ++r)
+        for (int r = 0; r < TILE_TOKENS; ++r)
             if (r < rows) store_f(out + ((size_t)(t0 + r) * heads + head) * width, c, acc[r]);
     }
+    if (blockIdx.z != 0) return;
     // the rotated part
-    for (int i = threadIdx.x; i < ABSORB_TOKENS * ((dr + 1) / 2); i += blockDim.x) {
+    for (int i = threadIdx.x; i < TILE_TOKENS * ((dr + 1) / 2); i += blockDim.x) {
         const int r = i / ((dr + 1) / 2), pair = i - r * ((dr + 1) / 2);
         if (r >= rows) continue;
         const size_t at = (size_t)(t0 + r) * q_row + head * (d + dr) + d + 2 * pair;
@@ -140,45 +182,39 @@ __global__ void latent_absorb_kernel(
     }
 }
 
-#define EXPAND_TOKENS 8
-
-// One workgroup a (tile of tokens, head).  w_uv_t is [heads][rank][dv] (transposed at load, so that lanes
-// read neighbouring numbers).  `lat` rows are `lat_row` wide, of which the first `rank` are read.
-// LDS: EXPAND_TOKENS * rank floats.
+// One workgroup a (tile of tokens, head, 64 value columns).  w_uv_t is [heads][rank][dv] (transposed at load, so that
+// lanes read neighbouring numbers).  `lat` rows are `lat_row` wide, of which the first `rank` are read.
+// LDS: TILE_TOKENS * rank floats, then the partial sums.
 template <typename TI, typename TW, typename TO>
-__global__ void latent_expand_kernel(
+__global__ void __launch_bounds__(TILE_WAVES * KIPP_WAVE) latent_expand_kernel(
     const TI* __restrict__ lat, int lat_row, const TW* __restrict__ w_uv_t, const float* __restrict__ gate, int gate_parts,
     size_t gate_part_stride, int gate_stride, TO* __restrict__ out, int n_tokens, int heads, int rank, int dv) {
-    extern __shared__ float l_s[];
-    const int t0 = blockIdx.x * EXPAND_TOKENS;
+    extern __shared__ float lds[];
+    float* l_s = lds;
+    float* red = lds + TILE_TOKENS * rank;
+    const int t0 = blockIdx.x * TILE_TOKENS;
     const int head = blockIdx.y;
-    const int rows = min(EXPAND_TOKENS, n_tokens - t0);
-    for (int i = threadIdx.x; i < EXPAND_TOKENS * rank; i += blockDim.x) {
+    const int rows = min(TILE_TOKENS, n_tokens - t0);
+    for (int i = threadIdx.x; i < TILE_TOKENS * rank; i += blockDim.x) {
         const int r = i / rank, e = i - r * rank;
         l_s[i] = r < rows ? load_f(lat, ((size_t)(t0 + r) * heads + head) * lat_row + e) : 0.0f;
     }
     __syncthreads();
-    const TW* w = w_uv_t + (size_t)head * rank * dv;
-    for (int c = threadIdx.x; c < dv; c += blockDim.x) {
-        float acc[EXPAND_TOKENS];
+    const int c = blockIdx.z * TILE_COLS + (threadIdx.x & (KIPP_WAVE - 1));
+    float acc[TILE_TOKENS];
+    tile_product(l_s, rank, w_uv_t + (size_t)head * rank * dv, dv, c, c < dv, acc);
+    tile_reduce(red, acc);
+    if (threadIdx.x >= KIPP_WAVE || c >= dv) return;
 #pragma unroll
-        for (int r = 0; r < EXPAND_TOKENS; ++r) acc[r] = 0.0f;
-        for (int e = 0; e < rank; ++e) {
-            const float wv = load_f(w, (size_t)e * dv + c);
-#pragma unroll
-            for (int r = 0; r < EXPAND_TOKENS; ++r) acc[r] = fmaf(l_s[r * rank + e], wv, acc[r]);
+    for (int r = 0; r < TILE_TOKENS; ++r) {
+        if (r >= rows) continue;
+        float g = 1.0f;
+        if (gate != nullptr) {
+            float z = 0.0f;
+            for (int p = 0; p < gate_parts; ++p) z += gate[p * gate_part_stride + (size_t)(t0 + r) * gate_stride + head];
+            g = 1.0f / (1.0f + expf(-z));
         }
-#pragma unroll
-        for (int r = 0; r < EXPAND_TOKENS; ++r) {
-            if (r >= rows) continue;
-            float g = 1.0f;
-            if (gate != nullptr) {
-                float z = 0.0f;
-                for (int p = 0; p < gate_parts; ++p) z += gate[p * gate_part_stride + (size_t)(t0 + r) * gate_stride + head];
-                g = 1.0f / (1.0f + expf(-z));
-            }
-            store_f(out + ((size_t)(t0 + r) * heads + head) * dv, c, acc[r] * g);
-        }
+        store_f(out + ((size_t)(t0 + r) * heads + head) * dv, c, acc[r] * g);
     }
 }
 
@@ -209,9 +245,9 @@ int kipp_latent_absorb(const float* q, int parts, const void* w_uk, int w_dtype,
                        int d, int dr, int rank, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (heads <= 0 || d <= 0 || dr < 0 || rank <= 0 || rot_dims > dr || rot_dims % 2) return -1;
-    const size_t lds = (size_t)ABSORB_TOKENS * d * sizeof(float);
+    const size_t lds = (size_t)(TILE_TOKENS * d + TILE_WAVES * TILE_TOKENS * TILE_COLS) * sizeof(float);
     if (lds > 64 * 1024) return -1;
-    dim3 grid((n_tokens + ABSORB_TOKENS - 1) / ABSORB_TOKENS, heads), block(rank >= 256 ? 256 : (rank >= 128 ? 128 : 64));
+    dim3 grid((n_tokens + TILE_TOKENS - 1) / TILE_TOKENS, heads, (rank + TILE_COLS - 1) / TILE_COLS), block(TILE_WAVES * KIPP_WAVE);
     const size_t part_stride = (size_t)n_tokens * heads * (d + dr);
 #define KIPP_LA(TW, TO)                                                                                                 \
     hipLaunchKernelGGL((latent_absorb_kernel<TW, TO>), grid, block, lds, stream, q, parts, part_stride, (const TW*)w_uk, \
@@ -228,9 +264,9 @@ int kipp_latent_expand(const void* lat, int lat_dtype, int lat_row, const void* 
                        hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (heads <= 0 || rank <= 0 || dv <= 0 || lat_row < rank) return -1;
-    const size_t lds = (size_t)EXPAND_TOKENS * rank * sizeof(float);
+    const size_t lds = (size_t)(TILE_TOKENS * rank + TILE_WAVES * TILE_TOKENS * TILE_COLS) * sizeof(float);
     if (lds > 64 * 1024) return -1;
-    dim3 grid((n_tokens + EXPAND_TOKENS - 1) / EXPAND_TOKENS, heads), block(dv >= 256 ? 256 : (dv >= 128 ? 128 : 64));
+    dim3 grid((n_tokens + TILE_TOKENS - 1) / TILE_TOKENS, heads, (dv + TILE_COLS - 1) / TILE_COLS), block(TILE_WAVES * KIPP_WAVE);
     const size_t gate_part_stride = (size_t)n_tokens * gate_stride;
 #define KIPP_LE(TI, TW, TO)                                                                                             \
     hipLaunchKernelGGL((latent_expand_kernel<TI, TW, TO>), grid, block, lds, stream, (const TI*)lat, lat_row,            \

@@ -8,16 +8,22 @@
 //     m' = max(lf + m, li)
 //     S' = exp(lf + m - m') S + exp(li - m') k v^T       (d x dv),   n' likewise with k alone
 //     o  = S'^T q / (max(|n' . q|, exp(-m')) + 1e-6)
-// S, n and m live in the request's state slot as float32 [heads][d][dv] | [Z][heads][d] | [Z][heads], Z = ceil(dv / columns of a workgroup):
+// S, n and m live in the request's state slot as float32 [heads][dv][d] | [Z][heads][d] | [Z][heads], Z = ceil(dv / columns of a workgroup)
+// (a column of S, the d numbers that meet one value, lies together):
 // every workgroup of a head keeps a copy of n and m of its own (all equal), so that none reads what another has
 // already written for the next step.  A slot that was just claimed holds zeros, which is the recurrence's start.
 // Everything here is float32.
 //
-// scan    a workgroup takes (entry of the batch, head, 64 columns of S) and walks the entry's tokens in order.
-//         A column is shared by 4 lanes that stand side by side in a wave, each with every fourth row of it, so
-//         the sum over rows ends in two lane exchanges and no wave waits for another: there is no barrier in
-//         the walk.  (Keys of more than 256 numbers: 16 lanes a column, 16 columns a workgroup.)  Every lane also keeps its rows of n (the same arithmetic in every column, hence the same
-//         bits), so the denominator needs no exchange between columns either.
+// scan    a workgroup takes (entry of the batch, head, a run of columns of S) and walks the entry's tokens in order.
+//         A column is shared by 4, 16 or 64 lanes that stand side by side in a wave, each with 8 (or 16) rows of it,
+//         so the sum over rows ends in a few lane exchanges and no wave waits for another inside the walk.  Every
+//         lane also keeps its rows of n (the same arithmetic in every column, hence the same bits), so the
+//         denominator needs no exchange between columns either.  The tokens come in chunks: while one chunk is
+//         walked out of LDS, the next one's k, q, v and gate pre-activations are on their way from memory into
+//         registers; tanh, logarithm and the first exponential of the gates are taken once a token by one lane when
+//         the chunk is put into LDS, so the walk itself is multiply-adds, one maximum and three exponentials a token.
+//         The order of a token's operations does not depend on where its chunk begins: a position's bits are the
+//         same however the prompt was cut.
 // finish  every head of a token divided by its root mean square, times the norm's weight, times sigmoid(gate),
 //         in the type the output projection reads.
 //
@@ -27,72 +33,174 @@
 #include <math.h>
 
 #define SCAN_THREADS 256
+#define SCAN_GROUP 8
+#define SCAN_STAGE 4096     // most numbers of k (and of q) that a chunk of tokens stages: 16 a thread
 
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.0f) - log1pf(expf(-fabsf(z))); }
 
-template <int ROWS, int SCAN_PARTS>     // rows of a column that one lane holds: ceil(d / SCAN_PARTS) <= ROWS
+// ROWS rows of a column a lane, PARTS lanes a column (side by side in a wave), 256 / PARTS columns a workgroup.
+// LDS: chunk * (2 d + columns + 2) floats.
+template <int ROWS, int PARTS>
 __global__ void __launch_bounds__(SCAN_THREADS) mlstm_scan_kernel(
     const float* __restrict__ proj, int stride, const float* __restrict__ bias_i, const float* __restrict__ bias_f, float cap,
     float* __restrict__ state, size_t state_stride, const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
-    const int32_t* __restrict__ slots, float* __restrict__ o_raw, int heads, int d, int dv) {
-    constexpr int SCAN_COLS = SCAN_THREADS / SCAN_PARTS;
-    const int seq = blockIdx.x, head = blockIdx.y;
-    const int part = threadIdx.x & (SCAN_PARTS - 1);
-    const int col = blockIdx.z * SCAN_COLS + threadIdx.x / SCAN_PARTS;
+    const int32_t* __restrict__ slots, float* __restrict__ o_raw, int heads, int d, int dv, int chunk) {
+    constexpr int COLS = SCAN_THREADS / PARTS;
+    constexpr int PER = SCAN_STAGE / SCAN_THREADS;          // staged numbers of k, and of q, a thread
+    constexpr int PER_V = 32 * COLS / SCAN_THREADS > 0 ? 32 * COLS / SCAN_THREADS : 1;
+    extern __shared__ float lds[];
+    float* k_s = lds;
+    float* q_s = k_s + (size_t)chunk * d;
+    float* v_s = q_s + (size_t)chunk * d;
+    float* li_s = v_s + (size_t)chunk * COLS;
+    float* lf_s = li_s + chunk;
+    const int seq = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
+    const int part = tid & (PARTS - 1), col_l = tid / PARTS;
+    const int col = blockIdx.z * COLS + col_l;
     const bool live = col < dv;
+    const int row0 = part * ROWS;
     const int first = q_start[seq], count = q_len[seq];
     float* slot = state + (size_t)slots[seq] * state_stride;
-    float* S_g = slot + (size_t)head * d * dv;
+    float* S_g = slot + ((size_t)head * dv + (live ? col : 0)) * d;
     float* n_g = slot + (size_t)heads * d * dv + ((size_t)blockIdx.z * heads + head) * d;
     float* m_g = slot + (size_t)heads * d * dv + (size_t)gridDim.z * heads * d + (size_t)blockIdx.z * heads + head;
 
     float S[ROWS], nv[ROWS];
+    // a lane's rows of a column lie together: 16 bytes a load where the addresses allow
+    const bool wide = d % 4 == 0 && (((uintptr_t)S_g | (uintptr_t)n_g) & 15) == 0 && row0 + ROWS <= d;
+    if (wide) {
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-        const int row = part + r * SCAN_PARTS;
-        S[r] = (live && row < d) ? S_g[(size_t)row * dv + col] : 0.0f;
-        nv[r] = row < d ? n_g[row] : 0.0f;
+        for (int r = 0; r < ROWS; r += 4) {
+            *reinterpret_cast<float4*>(S + r) = live ? *reinterpret_cast<const float4*>(S_g + row0 + r) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            *reinterpret_cast<float4*>(nv + r) = *reinterpret_cast<const float4*>(n_g + row0 + r);
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            const int row = row0 + r;
+            S[r] = (live && row < d) ? S_g[row] : 0.0f;
+            nv[r] = row < d ? n_g[row] : 0.0f;
+        }
     }
     float m = *m_g;
     const float q_scale = 1.0f / sqrtf((float)d);
     const float bi = bias_i[head], bf = bias_f[head];
-    const int at_k = heads * d, at_v = 2 * heads * d, at_i = 2 * heads * d + 2 * heads * dv, at_f = at_i + heads;
+    const int at_q = head * d, at_k = heads * d + head * d, at_v = 2 * heads * d + head * dv;
+    const int at_i = 2 * heads * d + 2 * heads * dv + head, at_f = at_i + heads;
 
-    for (int t = first; t < first + count; ++t) {
-        const float* row_p = proj + (size_t)t * stride;
-        const float li = cap * tanhf((row_p[at_i + head] + bi) / cap);
-        const float lf = log_sigmoid(cap * tanhf((row_p[at_f + head] + bf) / cap));
-        const float m_new = fmaxf(lf + m, li);
-        const float keep = expf(lf + m - m_new), take = expf(li - m_new);
-        const float v = live ? row_p[at_v + head * dv + col] : 0.0f;
-        float num = 0.0f, den = 0.0f;
+    // a chunk's numbers on their way: asked for before the chunk ahead of it is walked, put into LDS after
+    float k_r[PER], q_r[PER], v_r[PER_V], zi = 0.0f, zf = 0.0f;
+    auto fetch = [&](int c0, int n_tok) {
+        const float* base = proj + (size_t)(first + c0) * stride;
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int i = tid + j * SCAN_THREADS;
+            if (i < n_tok * d) {
+                const int tt = i / d, e = i - tt * d;
+                k_r[j] = base[(size_t)tt * stride + at_k + e];
+                q_r[j] = base[(size_t)tt * stride + at_q + e];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < PER_V; ++j) {
+            const int i = tid + j * SCAN_THREADS;
+            if (i < n_tok * COLS) {
+                const int tt = i / COLS, cc = blockIdx.z * COLS + (i - tt * COLS);
+                v_r[j] = cc < dv ? base[(size_t)tt * stride + at_v + cc] : 0.0f;
+            }
+        }
+        if (tid < n_tok) {
+            zi = base[(size_t)tid * stride + at_i];
+            zf = base[(size_t)tid * stride + at_f];
+        }
+    };
+    int n_tok = min(chunk, count);
+    fetch(0, n_tok);
+    for (int c0 = 0; c0 < count; c0 += chunk) {
+        __syncthreads();        // the chunk before has been walked by every wave
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int i = tid + j * SCAN_THREADS;
+            if (i < n_tok * d) {
+                k_s[i] = k_r[j];
+                q_s[i] = q_r[j] * q_scale;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < PER_V; ++j) {
+            const int i = tid + j * SCAN_THREADS;
+            if (i < n_tok * COLS) v_s[i] = v_r[j];
+        }
+        if (tid < n_tok) {      // the gates' logarithms, a lane a token; the walk below only takes maxima and exponentials
+            li_s[tid] = cap * tanhf((zi + bi) / cap);
+            lf_s[tid] = log_sigmoid(cap * tanhf((zf + bf) / cap));
+        }
+        __syncthreads();
+        const int n_next = min(chunk, count - c0 - chunk);
+        if (n_next > 0) fetch(c0 + chunk, n_next);
+        // eight tokens at a time: their sums over a lane's rows first, then the exchanges between the lanes of a
+        // column for all eight together (each exchange waits as long as a read of LDS; eight of them wait together)
+        for (int t8 = 0; t8 < n_tok; t8 += SCAN_GROUP) {
+            float num_p[SCAN_GROUP], den_p[SCAN_GROUP], floor_p[SCAN_GROUP];
+#pragma unroll
+            for (int u = 0; u < SCAN_GROUP; ++u) {
+                const int tt = t8 + u;
+                num_p[u] = den_p[u] = floor_p[u] = 0.0f;
+                if (tt < n_tok) {
+                    const float li = li_s[tt], lf = lf_s[tt];
+                    const float m_new = fmaxf(lf + m, li);
+                    const float keep = expf(lf + m - m_new), take = expf(li - m_new);
+                    const float tv = take * v_s[tt * COLS + col_l];
+                    const float* k_t = k_s + (size_t)tt * d + row0;
+                    const float* q_t = q_s + (size_t)tt * d + row0;
+                    float num = 0.0f, den = 0.0f;
+#pragma unroll
+                    for (int r = 0; r < ROWS; ++r) {
+                        const bool in = row0 + r < d;
+                        const float k = in ? k_t[r] : 0.0f, q = in ? q_t[r] : 0.0f;
+                        S[r] = fmaf(keep, S[r], k * tv);
+                        nv[r] = fmaf(keep, nv[r], take * k);
+                        num = fmaf(S[r], q, num);
+                        den = fmaf(nv[r], q, den);
+                    }
+                    m = m_new;
+                    num_p[u] = num;
+                    den_p[u] = den;
+                    floor_p[u] = expf(-m);
+                }
+            }
+#pragma unroll
+            for (int off = 1; off < PARTS; off <<= 1) {
+#pragma unroll
+                for (int u = 0; u < SCAN_GROUP; ++u) {
+                    num_p[u] += __shfl_xor(num_p[u], off, KIPP_WAVE);
+                    den_p[u] += __shfl_xor(den_p[u], off, KIPP_WAVE);
+                }
+            }
+            if (live && part == 0) {
+#pragma unroll
+                for (int u = 0; u < SCAN_GROUP; ++u)
+                    if (t8 + u < n_tok)
+                        o_raw[((size_t)(first + c0 + t8 + u) * heads + head) * dv + col] = num_p[u] / (fmaxf(fabsf(den_p[u]), floor_p[u]) + 1e-6f);
+            }
+        }
+        n_tok = n_next;
+    }
+    if (wide) {
+#pragma unroll
+        for (int r = 0; r < ROWS; r += 4) {
+            if (live) *reinterpret_cast<float4*>(S_g + row0 + r) = *reinterpret_cast<float4*>(S + r);
+            if (col_l == 0) *reinterpret_cast<float4*>(n_g + row0 + r) = *reinterpret_cast<float4*>(nv + r);
+        }
+    } else {
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) {
-            const int row = part + r * SCAN_PARTS;
-            const float k = row < d ? row_p[at_k + head * d + row] : 0.0f;
-            const float q = row < d ? row_p[head * d + row] * q_scale : 0.0f;
-            const float tk = take * k;
-            S[r] = fmaf(keep, S[r], tk * v);
-            nv[r] = fmaf(keep, nv[r], tk);
-            num = fmaf(S[r], q, num);
-            den = fmaf(nv[r], q, den);
+            const int row = row0 + r;
+            if (live && row < d) S_g[row] = S[r];
+            if (col_l == 0 && row < d) n_g[row] = nv[r];
         }
-#pragma unroll
-        for (int off = 1; off < SCAN_PARTS; off <<= 1) {
-            num += __shfl_xor(num, off, KIPP_WAVE);
-            den += __shfl_xor(den, off, KIPP_WAVE);
-        }
-        m = m_new;
-        if (live && part == 0)
-            o_raw[((size_t)t * heads + head) * dv + col] = num / (fmaxf(fabsf(den), expf(-m)) + 1e-6f);
     }
-#pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-        const int row = part + r * SCAN_PARTS;
-        if (live && row < d) S_g[(size_t)row * dv + col] = S[r];
-        if (threadIdx.x < SCAN_PARTS && row < d) n_g[row] = nv[r];
-    }
-    if (threadIdx.x == 0) *m_g = m;
+    if (tid == 0) *m_g = m;
 }
 
 #define FINISH_HEADS 4
@@ -114,6 +222,9 @@ __global__ void mlstm_finish_kernel(const float* __restrict__ o_raw, const float
         store_f(dst, e, src[e] * scale * norm_w[head * dv + e] * (1.0f / (1.0f + expf(-gate[e]))));
 }
 
+// Lanes that share a column of the memory: 8 rows a lane (16 for keys of more than 512 numbers).
+static int kipp_mlstm_parts(int d) { return d <= 32 ? 4 : (d <= 128 ? 16 : 64); }
+
 extern "C" {
 
 int kipp_mlstm_scan(const float* proj, int stride, const float* bias_i, const float* bias_f, float cap, float* state,
@@ -121,20 +232,20 @@ int kipp_mlstm_scan(const float* proj, int stride, const float* bias_i, const fl
                     int n_seqs, int heads, int d, int dv, hipStream_t stream) {
     if (n_seqs <= 0) return 0;
     if (heads <= 0 || d <= 0 || d > 1024 || dv <= 0 || !(cap > 0.0f)) return -1;
-    const int parts = d <= 256 ? 4 : 16;
+    const int parts = kipp_mlstm_parts(d);
     const int cols = SCAN_THREADS / parts;
     if (stride < 2 * heads * d + 2 * heads * dv + 2 * heads || state_stride < (size_t)heads * d * dv + (size_t)((dv + cols - 1) / cols) * (heads * d + heads)) return -1;
     dim3 grid(n_seqs, heads, (dv + cols - 1) / cols), block(SCAN_THREADS);
-    const int rows = (d + parts - 1) / parts;
-#define KIPP_SCAN(R, P)                                                                                                        \
-    hipLaunchKernelGGL((mlstm_scan_kernel<R, P>), grid, block, 0, stream, proj, stride, bias_i, bias_f, cap, state, state_stride, \
-                       q_start, q_len, slots, o_raw, heads, d, dv)
-    if (parts == 16) KIPP_SCAN(64, 16);
-    else if (rows <= 4) KIPP_SCAN(4, 4);
-    else if (rows <= 8) KIPP_SCAN(8, 4);
-    else if (rows <= 16) KIPP_SCAN(16, 4);
-    else if (rows <= 32) KIPP_SCAN(32, 4);
-    else KIPP_SCAN(64, 4);
+    int chunk = SCAN_STAGE / d;                       // tokens whose k and q fit the staging registers
+    if (chunk > 32) chunk = 32;
+    const size_t lds = (size_t)chunk * (2 * d + cols + 2) * sizeof(float);
+#define KIPP_SCAN(R, P)                                                                                                          \
+    hipLaunchKernelGGL((mlstm_scan_kernel<R, P>), grid, block, lds, stream, proj, stride, bias_i, bias_f, cap, state, state_stride, \
+                       q_start, q_len, slots, o_raw, heads, d, dv, chunk)
+    if (parts == 4) KIPP_SCAN(8, 4);
+    else if (parts == 16) KIPP_SCAN(8, 16);
+    else if (d <= 512) KIPP_SCAN(8, 64);
+    else KIPP_SCAN(16, 64);
 #undef KIPP_SCAN
     return KIPP_LAUNCH_CHECK();
 }

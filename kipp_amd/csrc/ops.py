@@ -488,7 +488,7 @@ def latent_absorb(q: torch.Tensor, w_uk: torch.Tensor, out: torch.Tensor, positi
     _need(stride == heads * (d + dr) and out.shape == (n, heads * (rank + dr)) and positions.numel() == n,
           "latent_absorb: q is [tokens, heads (d + dr)], out [tokens, heads (rank + dr)]")
     _need(w_uk.shape == (heads * d, rank) and _code(w_uk) == _code(out), "latent_absorb: w_uk is [heads d, rank] in the output's type")
-    _need(d * 32 <= 64 * 1024, "latent_absorb: unrotated head size too large")
+    _need(d * 32 + 8192 <= 64 * 1024, "latent_absorb: unrotated head size too large")
     fn = _fn("latent", "kipp_latent_absorb", [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_float]
              + [_c_int] * 5 + [_c_ptr])
     _check(fn(_ptr(q), parts, _ptr(w_uk), _code(w_uk), _ptr(out), _code(out), _ptr(positions), _ptr(freq), int(rot_dims),
@@ -506,7 +506,7 @@ def latent_expand(lat: torch.Tensor, w_uv_t: torch.Tensor, out: torch.Tensor, he
     _need(lat.dim() == 2 and lat.shape[1] % heads == 0 and lat.shape[1] // heads >= rank, "latent_expand: lat is [tokens, heads row]")
     _need(w_uv_t.shape == (heads, rank, dv) and out.shape == (n, heads * dv) and _code(lat) == _code(w_uv_t) == _code(out),
           "latent_expand: w_uv_t is [heads, rank, dv]; one type")
-    _need(rank * 32 <= 64 * 1024, "latent_expand: latent too wide")
+    _need(rank * 32 + 8192 <= 64 * 1024, "latent_expand: latent too wide")
     g_parts, g_stride, g_ptr = 0, 0, None
     if gate is not None:
         g_parts, g_n, g_stride = _slabs(gate, "latent_expand")
@@ -523,13 +523,14 @@ def latent_expand(lat: torch.Tensor, w_uv_t: torch.Tensor, out: torch.Tensor, he
 
 def mlstm_columns(d: int) -> int:
     """Columns of the memory that a workgroup of the scan takes (fewer where a column's rows need more lanes)."""
-    return 64 if d <= 256 else 16
+    return 256 // (4 if d <= 32 else (16 if d <= 128 else 64))
 
 
 def mlstm_state_size(heads: int, d: int, dv: int) -> int:
-    """float32 numbers of a request's state: S [heads, d, dv], then a copy of n [heads, d] and m [heads] for every
+    """float32 numbers of a request's state: S [heads, dv, d], then a copy of n [heads, d] and m [heads] for every
     workgroup's columns."""
-    return heads * d * dv + -(-dv // mlstm_columns(d)) * (heads * d + heads)
+    size = heads * d * dv + -(-dv // mlstm_columns(d)) * (heads * d + heads)
+    return -(-size // 4) * 4       # slots begin at multiples of 16 bytes
 
 
 def mlstm_scan(proj: torch.Tensor, bias_i: torch.Tensor, bias_f: torch.Tensor, cap: float, state: torch.Tensor,

@@ -45,8 +45,11 @@ __device__ __forceinline__ void load_coefficients(StreamCoefficients& c, const f
     }
 }
 
-// write (if mix != nullptr), then read and norm (if inw != nullptr).  LDS: width floats + 16.
-template <typename TO>
+// write (if mix != nullptr), then read and norm (if inw != nullptr).  R copies (a build constant where it is 1 to 4, so
+// that the coefficients and a lane's rows stay in registers), VEC numbers a lane and load (4 where the width
+// allows); the workgroup is sized so that a lane meets its numbers once where the width allows, with every load
+// of a token asked for before the first is used.  LDS: width floats + 16.
+template <int RMAX, int VEC, typename TO>
 __global__ void streams_step_kernel(float* __restrict__ X, const float* __restrict__ delta, int parts, size_t part_stride,
                                     const float* __restrict__ mix, const float* __restrict__ outw,
                                     const float* __restrict__ inw, const float* __restrict__ norm_w, float eps,
@@ -55,46 +58,75 @@ __global__ void streams_step_kernel(float* __restrict__ X, const float* __restri
     float* u_s = lds + 16;
     const int t = blockIdx.x;
     float* rows = X + (size_t)t * R * width;
-    StreamCoefficients c;
-    load_coefficients(c, mix, outw, inw, R);
+    float c_mix[RMAX][RMAX], c_out[RMAX], c_in[RMAX];
+#pragma unroll
+    for (int s = 0; s < RMAX; ++s) {
+#pragma unroll
+        for (int to = 0; to < RMAX; ++to) c_mix[s][to] = (mix != nullptr && s < R && to < R) ? mix[s * R + to] : 0.0f;
+        c_out[s] = (outw != nullptr && s < R) ? outw[s] : 0.0f;
+        c_in[s] = (inw != nullptr && s < R) ? inw[s] : 0.0f;
+    }
     float ss = 0.0f;
-    for (int e = threadIdx.x; e < width; e += blockDim.x) {
-        float x[STREAMS_MAX];
+    for (int e = threadIdx.x * VEC; e < width; e += blockDim.x * VEC) {
+        float x[RMAX][VEC], y[VEC];
 #pragma unroll
-        for (int r = 0; r < STREAMS_MAX; ++r) x[r] = r < R ? rows[(size_t)r * width + e] : 0.0f;
+        for (int r = 0; r < RMAX; ++r) {
+            if (r < R) {
+                if (VEC == 4) *reinterpret_cast<float4*>(x[r]) = *reinterpret_cast<const float4*>(rows + (size_t)r * width + e);
+                else x[r][0] = rows[(size_t)r * width + e];
+            } else {
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) x[r][v] = 0.0f;
+            }
+        }
         if (mix != nullptr) {
-            float y = 0.0f;
-            for (int p = 0; p < parts; ++p) y += delta[p * part_stride + (size_t)t * width + e];
-            float fresh[STREAMS_MAX];
 #pragma unroll
-            for (int to = 0; to < STREAMS_MAX; ++to) {
-                float v = 0.0f;
-                if (to < R) {
+            for (int v = 0; v < VEC; ++v) y[v] = 0.0f;
+            for (int p = 0; p < parts; ++p) {
+                float d4[VEC];
+                if (VEC == 4) *reinterpret_cast<float4*>(d4) = *reinterpret_cast<const float4*>(delta + p * part_stride + (size_t)t * width + e);
+                else d4[0] = delta[p * part_stride + (size_t)t * width + e];
 #pragma unroll
-                    for (int s = 0; s < STREAMS_MAX; ++s)
-                        if (s < R) v += c.mix[s][to] * x[s];
-                    v += c.out[to] * y;
-                    rows[(size_t)to * width + e] = v;
+                for (int v = 0; v < VEC; ++v) y[v] += d4[v];
+            }
+            float fresh[RMAX][VEC];
+#pragma unroll
+            for (int to = 0; to < RMAX; ++to) {
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) {
+                    float acc = 0.0f;
+#pragma unroll
+                    for (int s = 0; s < RMAX; ++s) acc += c_mix[s][to] * x[s][v];
+                    fresh[to][v] = acc + c_out[to] * y[v];
                 }
-                fresh[to] = v;
+                if (to < R) {
+                    if (VEC == 4) *reinterpret_cast<float4*>(rows + (size_t)to * width + e) = *reinterpret_cast<float4*>(fresh[to]);
+                    else rows[(size_t)to * width + e] = fresh[to][0];
+                }
             }
 #pragma unroll
-            for (int r = 0; r < STREAMS_MAX; ++r) x[r] = fresh[r];
+            for (int r = 0; r < RMAX; ++r)
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) x[r][v] = fresh[r][v];
         }
         if (inw != nullptr) {
-            float u = 0.0f;
 #pragma unroll
-            for (int r = 0; r < STREAMS_MAX; ++r)
-                if (r < R) u += c.in[r] * x[r];
-            u_s[e] = u;
-            ss = fmaf(u, u, ss);
+            for (int v = 0; v < VEC; ++v) {
+                float u = 0.0f;
+#pragma unroll
+                for (int r = 0; r < RMAX; ++r) u += c_in[r] * x[r][v];
+                u_s[e + v] = u;
+                ss = fmaf(u, u, ss);
+            }
         }
     }
     if (inw == nullptr) return;
     ss = block_sum(ss, lds);
     const float scale = 1.0f / sqrtf(ss / (float)width + eps);
     TO* dst = h + (size_t)t * width;
-    for (int e = threadIdx.x; e < width; e += blockDim.x) store_f(dst, e, u_s[e] * scale * norm_w[e]);
+    for (int e = threadIdx.x * VEC; e < width; e += blockDim.x * VEC)
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) store_f(dst, e + v, u_s[e + v] * scale * norm_w[e + v]);
 }
 
 __global__ void streams_close_kernel(const float* __restrict__ X, const float* __restrict__ delta, int parts, size_t part_stride,
@@ -156,12 +188,26 @@ int kipp_streams_step(float* X, const float* delta, int parts, const float* mix,
     if (inw != nullptr && (norm_w == nullptr || h == nullptr)) return -2;
     const size_t lds = (size_t)(width + 16) * sizeof(float);
     const size_t stride = (size_t)n * width;
-    if (h_dtype == KIPP_BF16)
-        hipLaunchKernelGGL(streams_step_kernel<bf16_t>, dim3(n), dim3(block_for(width)), lds, stream, X, delta, parts, stride, mix, outw,
-                           inw, norm_w, eps, (bf16_t*)h, R, width);
-    else
-        hipLaunchKernelGGL(streams_step_kernel<float>, dim3(n), dim3(block_for(width)), lds, stream, X, delta, parts, stride, mix, outw,
-                           inw, norm_w, eps, (float*)h, R, width);
+    const bool wide = width % 4 == 0 && (((uintptr_t)X | (uintptr_t)delta) & 15) == 0;
+    const int lanes = wide ? width / 4 : width;
+    const int threads = lanes >= 1024 ? 1024 : ((lanes + KIPP_WAVE - 1) / KIPP_WAVE) * KIPP_WAVE;
+#define KIPP_SS(RMAX, VEC, TO)                                                                                                  \
+    hipLaunchKernelGGL((streams_step_kernel<RMAX, VEC, TO>), dim3(n), dim3(threads), lds, stream, X, delta, parts, stride, mix, \
+                       outw, inw, norm_w, eps, (TO*)h, R, width)
+#define KIPP_SS_R(VEC, TO)                   \
+    do {                                     \
+        if (R == 1) KIPP_SS(1, VEC, TO);     \
+        else if (R == 2) KIPP_SS(2, VEC, TO); \
+        else if (R <= 4) KIPP_SS(4, VEC, TO); \
+        else KIPP_SS(STREAMS_MAX, VEC, TO);  \
+    } while (0)
+    if (h_dtype == KIPP_BF16) {
+        if (wide) KIPP_SS_R(4, bf16_t); else KIPP_SS_R(1, bf16_t);
+    } else {
+        if (wide) KIPP_SS_R(4, float); else KIPP_SS_R(1, float);
+    }
+#undef KIPP_SS_R
+#undef KIPP_SS
     return KIPP_LAUNCH_CHECK();
 }
 

@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 SHAPES = ("rerizen-tiny-a", "rerizen-tiny-b")
 LENGTHS = [1, 19, 45, 80, 131]
-TOL = {"float32": 1e-9, "bfloat16": 1.5e-3}     # float32 is the sharp test; narrow widths make bfloat16 rows noisy
+TOL = {"float32": 1e-9, "bfloat16": 3e-3}     # float32 is the sharp test; narrow widths make bfloat16 rows noisy
 
 
 @pytest.fixture(scope="module")
