@@ -38,20 +38,22 @@
 
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.0f) - log1pf(expf(-fabsf(z))); }
 
-// ROWS rows of a column a lane, PARTS lanes a column (side by side in a wave), 256 / PARTS columns a workgroup.
-// LDS: chunk * (2 d + columns + 2) floats.
+// ROWS rows of a column a lane (a multiple of 4), PARTS lanes a column (side by side in a wave), 256 / PARTS columns a
+// workgroup.  `unit`: columns that share one copy of n and m in the state (a workgroup's columns are a multiple of it).
+// LDS: chunk * (2 ROWS PARTS + columns + 2) floats; rows of k and q are padded with zeros to ROWS * PARTS numbers.
 template <int ROWS, int PARTS>
 __global__ void __launch_bounds__(SCAN_THREADS) mlstm_scan_kernel(
     const float* __restrict__ proj, int stride, const float* __restrict__ bias_i, const float* __restrict__ bias_f, float cap,
     float* __restrict__ state, size_t state_stride, const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
-    const int32_t* __restrict__ slots, float* __restrict__ o_raw, int heads, int d, int dv, int chunk) {
+    const int32_t* __restrict__ slots, float* __restrict__ o_raw, int heads, int d, int dv, int chunk, int unit, int copies) {
     constexpr int COLS = SCAN_THREADS / PARTS;
+    constexpr int DP = ROWS * PARTS;                        // a staged row of k or q
     constexpr int PER = SCAN_STAGE / SCAN_THREADS;          // staged numbers of k, and of q, a thread
     constexpr int PER_V = 32 * COLS / SCAN_THREADS > 0 ? 32 * COLS / SCAN_THREADS : 1;
-    extern __shared__ float lds[];
+    extern __shared__ __align__(16) float lds[];
     float* k_s = lds;
-    float* q_s = k_s + (size_t)chunk * d;
-    float* v_s = q_s + (size_t)chunk * d;
+    float* q_s = k_s + (size_t)chunk * DP;
+    float* v_s = q_s + (size_t)chunk * DP;
     float* li_s = v_s + (size_t)chunk * COLS;
     float* lf_s = li_s + chunk;
     const int seq = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
@@ -62,12 +64,16 @@ __global__ void __launch_bounds__(SCAN_THREADS) mlstm_scan_kernel(
     const int first = q_start[seq], count = q_len[seq];
     float* slot = state + (size_t)slots[seq] * state_stride;
     float* S_g = slot + ((size_t)head * dv + (live ? col : 0)) * d;
-    float* n_g = slot + (size_t)heads * d * dv + ((size_t)blockIdx.z * heads + head) * d;
-    float* m_g = slot + (size_t)heads * d * dv + (size_t)gridDim.z * heads * d + (size_t)blockIdx.z * heads + head;
+    float* n_all = slot + (size_t)heads * d * dv;
+    float* m_all = n_all + (size_t)copies * heads * d;
+    const int copy_in = blockIdx.z * COLS / unit;            // every copy holds the same numbers: the first of this workgroup's is read
+    const float* n_g = n_all + ((size_t)copy_in * heads + head) * d;
+    const bool writes_copy = live && col % unit == 0;       // this column's lanes write the copy of the column's unit
+    float* n_w = n_all + ((size_t)((live ? col : 0) / unit) * heads + head) * d;
 
     float S[ROWS], nv[ROWS];
     // a lane's rows of a column lie together: 16 bytes a load where the addresses allow
-    const bool wide = d % 4 == 0 && (((uintptr_t)S_g | (uintptr_t)n_g) & 15) == 0 && row0 + ROWS <= d;
+    const bool wide = d % 4 == 0 && (((uintptr_t)S_g | (uintptr_t)n_g | (uintptr_t)n_w) & 15) == 0 && row0 + ROWS <= d;
     if (wide) {
 #pragma unroll
         for (int r = 0; r < ROWS; r += 4) {
@@ -82,7 +88,7 @@ __global__ void __launch_bounds__(SCAN_THREADS) mlstm_scan_kernel(
             nv[r] = row < d ? n_g[row] : 0.0f;
         }
     }
-    float m = *m_g;
+    float m = m_all[(size_t)copy_in * heads + head];
     const float q_scale = 1.0f / sqrtf((float)d);
     const float bi = bias_i[head], bf = bias_f[head];
     const int at_q = head * d, at_k = heads * d + head * d, at_v = 2 * heads * d + head * dv;
@@ -95,10 +101,13 @@ __global__ void __launch_bounds__(SCAN_THREADS) mlstm_scan_kernel(
 #pragma unroll
         for (int j = 0; j < PER; ++j) {
             const int i = tid + j * SCAN_THREADS;
-            if (i < n_tok * d) {
-                const int tt = i / d, e = i - tt * d;
-                k_r[j] = base[(size_t)tt * stride + at_k + e];
-                q_r[j] = base[(size_t)tt * stride + at_q + e];
+            k_r[j] = q_r[j] = 0.0f;
+            if (i < n_tok * DP) {
+                const int tt = i / DP, e = i - tt * DP;
+                if (e < d) {
+                    k_r[j] = base[(size_t)tt * stride + at_k + e];
+                    q_r[j] = base[(size_t)tt * stride + at_q + e];
+                }
             }
         }
 #pragma unroll
@@ -121,7 +130,7 @@ __global__ void __launch_bounds__(SCAN_THREADS) mlstm_scan_kernel(
 #pragma unroll
         for (int j = 0; j < PER; ++j) {
             const int i = tid + j * SCAN_THREADS;
-            if (i < n_tok * d) {
+            if (i < n_tok * DP) {
                 k_s[i] = k_r[j];
                 q_s[i] = q_r[j] * q_scale;
             }
@@ -138,35 +147,50 @@ __global__ void __launch_bounds__(SCAN_THREADS) mlstm_scan_kernel(
         __syncthreads();
         const int n_next = min(chunk, count - c0 - chunk);
         if (n_next > 0) fetch(c0 + chunk, n_next);
-        // eight tokens at a time: their sums over a lane's rows first, then the exchanges between the lanes of a
-        // column for all eight together (each exchange waits as long as a read of LDS; eight of them wait together)
+        // eight tokens at a time: the gates' chain first (one maximum and three exponentials a token, no lane waits for
+        // another), then the multiply-adds over a lane's rows, then the exchanges between the lanes of a column for all
+        // eight together (each exchange waits as long as a read of LDS; eight of them wait together)
         for (int t8 = 0; t8 < n_tok; t8 += SCAN_GROUP) {
-            float num_p[SCAN_GROUP], den_p[SCAN_GROUP], floor_p[SCAN_GROUP];
+            float keep[SCAN_GROUP], take[SCAN_GROUP], floor_p[SCAN_GROUP], num_p[SCAN_GROUP], den_p[SCAN_GROUP];
 #pragma unroll
             for (int u = 0; u < SCAN_GROUP; ++u) {
-                const int tt = t8 + u;
-                num_p[u] = den_p[u] = floor_p[u] = 0.0f;
-                if (tt < n_tok) {
-                    const float li = li_s[tt], lf = lf_s[tt];
-                    const float m_new = fmaxf(lf + m, li);
-                    const float keep = expf(lf + m - m_new), take = expf(li - m_new);
-                    const float tv = take * v_s[tt * COLS + col_l];
-                    const float* k_t = k_s + (size_t)tt * d + row0;
-                    const float* q_t = q_s + (size_t)tt * d + row0;
-                    float num = 0.0f, den = 0.0f;
+                const int tt = min(t8 + u, n_tok - 1);
+                const float li = li_s[tt], lf = lf_s[tt];
+                const float m_new = t8 + u < n_tok ? fmaxf(lf + m, li) : m;
+                keep[u] = expf(lf + m - m_new);
+                take[u] = expf(li - m_new);
+                floor_p[u] = expf(-m_new);
+                m = m_new;
+            }
+#pragma unroll
+            for (int u = 0; u < SCAN_GROUP; ++u) {
+                num_p[u] = den_p[u] = 0.0f;
+                if (t8 + u < n_tok) {
+                    const int tt = t8 + u;
+                    const float tv = take[u] * v_s[tt * COLS + col_l];
+                    const float* k_t = k_s + (size_t)tt * DP + row0;
+                    const float* q_t = q_s + (size_t)tt * DP + row0;
+                    float kk[ROWS], qq[ROWS];
+#pragma unroll
+                    for (int r = 0; r < ROWS; r += 4) {
+                        *reinterpret_cast<float4*>(kk + r) = *reinterpret_cast<const float4*>(k_t + r);
+                        *reinterpret_cast<float4*>(qq + r) = *reinterpret_cast<const float4*>(q_t + r);
+                    }
+                    // rows are summed in runs of 8 and the runs pairwise, as the lanes of the 8-row build add theirs:
+                    // the build with 32 rows a lane (few tokens an entry) gives the same bits
+                    constexpr int RUNS = ROWS == 32 ? 4 : 1;
+                    float num[RUNS], den[RUNS];
+#pragma unroll
+                    for (int g = 0; g < RUNS; ++g) num[g] = den[g] = 0.0f;
 #pragma unroll
                     for (int r = 0; r < ROWS; ++r) {
-                        const bool in = row0 + r < d;
-                        const float k = in ? k_t[r] : 0.0f, q = in ? q_t[r] : 0.0f;
-                        S[r] = fmaf(keep, S[r], k * tv);
-                        nv[r] = fmaf(keep, nv[r], take * k);
-                        num = fmaf(S[r], q, num);
-                        den = fmaf(nv[r], q, den);
+                        S[r] = fmaf(keep[u], S[r], kk[r] * tv);
+                        nv[r] = fmaf(keep[u], nv[r], take[u] * kk[r]);
+                        num[r / (ROWS / RUNS)] = fmaf(S[r], qq[r], num[r / (ROWS / RUNS)]);
+                        den[r / (ROWS / RUNS)] = fmaf(nv[r], qq[r], den[r / (ROWS / RUNS)]);
                     }
-                    m = m_new;
-                    num_p[u] = num;
-                    den_p[u] = den;
-                    floor_p[u] = expf(-m);
+                    num_p[u] = RUNS == 4 ? (num[0] + num[1]) + (num[RUNS / 2] + num[RUNS - 1]) : num[0];
+                    den_p[u] = RUNS == 4 ? (den[0] + den[1]) + (den[RUNS / 2] + den[RUNS - 1]) : den[0];
                 }
             }
 #pragma unroll
@@ -190,17 +214,17 @@ __global__ void __launch_bounds__(SCAN_THREADS) mlstm_scan_kernel(
 #pragma unroll
         for (int r = 0; r < ROWS; r += 4) {
             if (live) *reinterpret_cast<float4*>(S_g + row0 + r) = *reinterpret_cast<float4*>(S + r);
-            if (col_l == 0) *reinterpret_cast<float4*>(n_g + row0 + r) = *reinterpret_cast<float4*>(nv + r);
+            if (writes_copy) *reinterpret_cast<float4*>(n_w + row0 + r) = *reinterpret_cast<float4*>(nv + r);
         }
     } else {
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) {
             const int row = row0 + r;
             if (live && row < d) S_g[row] = S[r];
-            if (col_l == 0 && row < d) n_g[row] = nv[r];
+            if (writes_copy && row < d) n_w[row] = nv[r];
         }
     }
-    if (tid == 0) *m_g = m;
+    if (writes_copy && part == 0) m_all[(size_t)(col / unit) * heads + head] = m;
 }
 
 #define FINISH_HEADS 4
@@ -222,29 +246,36 @@ __global__ void mlstm_finish_kernel(const float* __restrict__ o_raw, const float
         store_f(dst, e, src[e] * scale * norm_w[head * dv + e] * (1.0f / (1.0f + expf(-gate[e]))));
 }
 
-// Lanes that share a column of the memory: 8 rows a lane (16 for keys of more than 512 numbers).
+// Lanes that share a column of the memory in the walk over prompt portions: 8 rows a lane (16 for keys of more than
+// 512 numbers).  256 / lanes is the `unit`: the columns that share a copy of n and m in the state.
 static int kipp_mlstm_parts(int d) { return d <= 32 ? 4 : (d <= 128 ? 16 : 64); }
 
 extern "C" {
 
+// `few`: every entry brings few tokens (single decoded tokens): where the key size allows, a workgroup takes 64 columns
+// with 4 lanes each, a quarter of the workgroups, each reading longer runs of the state.
 int kipp_mlstm_scan(const float* proj, int stride, const float* bias_i, const float* bias_f, float cap, float* state,
                     size_t state_stride, const int32_t* q_start, const int32_t* q_len, const int32_t* slots, float* o_raw,
-                    int n_seqs, int heads, int d, int dv, hipStream_t stream) {
+                    int n_seqs, int heads, int d, int dv, int few, hipStream_t stream) {
     if (n_seqs <= 0) return 0;
     if (heads <= 0 || d <= 0 || d > 1024 || dv <= 0 || !(cap > 0.0f)) return -1;
-    const int parts = kipp_mlstm_parts(d);
+    const int unit = SCAN_THREADS / kipp_mlstm_parts(d);
+    const int copies = (dv + unit - 1) / unit;
+    if (stride < 2 * heads * d + 2 * heads * dv + 2 * heads || state_stride < (size_t)heads * d * dv + (size_t)copies * (heads * d + heads)) return -1;
+    const int parts = (few && d > 32 && d <= 128) ? 4 : kipp_mlstm_parts(d);
+    const int rows = parts == 4 ? (d <= 32 ? 8 : 32) : (d <= 512 ? 8 : 16);
     const int cols = SCAN_THREADS / parts;
-    if (stride < 2 * heads * d + 2 * heads * dv + 2 * heads || state_stride < (size_t)heads * d * dv + (size_t)((dv + cols - 1) / cols) * (heads * d + heads)) return -1;
     dim3 grid(n_seqs, heads, (dv + cols - 1) / cols), block(SCAN_THREADS);
-    int chunk = SCAN_STAGE / d;                       // tokens whose k and q fit the staging registers
+    int chunk = SCAN_STAGE / (rows * parts);          // tokens whose k and q fit the staging registers
     if (chunk > 32) chunk = 32;
-    const size_t lds = (size_t)chunk * (2 * d + cols + 2) * sizeof(float);
+    const size_t lds = (size_t)chunk * (2 * rows * parts + cols + 2) * sizeof(float);
 #define KIPP_SCAN(R, P)                                                                                                          \
     hipLaunchKernelGGL((mlstm_scan_kernel<R, P>), grid, block, lds, stream, proj, stride, bias_i, bias_f, cap, state, state_stride, \
-                       q_start, q_len, slots, o_raw, heads, d, dv, chunk)
-    if (parts == 4) KIPP_SCAN(8, 4);
+                       q_start, q_len, slots, o_raw, heads, d, dv, chunk, unit, copies)
+    if (parts == 4 && rows == 8) KIPP_SCAN(8, 4);
+    else if (parts == 4) KIPP_SCAN(32, 4);
     else if (parts == 16) KIPP_SCAN(8, 16);
-    else if (d <= 512) KIPP_SCAN(8, 64);
+    else if (rows == 8) KIPP_SCAN(8, 64);
     else KIPP_SCAN(16, 64);
 #undef KIPP_SCAN
     return KIPP_LAUNCH_CHECK();

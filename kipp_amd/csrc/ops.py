@@ -535,9 +535,9 @@ def mlstm_state_size(heads: int, d: int, dv: int) -> int:
 
 def mlstm_scan(proj: torch.Tensor, bias_i: torch.Tensor, bias_f: torch.Tensor, cap: float, state: torch.Tensor,
                q_start: torch.Tensor, q_len: torch.Tensor, slots: torch.Tensor, o_raw: torch.Tensor,
-               heads: int, d: int, dv: int) -> torch.Tensor:
+               heads: int, d: int, dv: int, few: bool = False) -> torch.Tensor:
     """The recurrence over every entry's tokens, in order, from and into the entry's slot of `state` [slots, size]
-    (float32).  `proj`: float32 [tokens, >= 2 heads d + 2 heads dv + 2 heads], columns q | k | v | gate | zi | zf;
+    (float32).  `few`: every entry brings few tokens (single decoded tokens): fewer, larger workgroups; the same bits.  `proj`: float32 [tokens, >= 2 heads d + 2 heads dv + 2 heads], columns q | k | v | gate | zi | zf;
     `o_raw` float32 [tokens, heads dv] receives S^T q over its denominator."""
     _dev(proj, bias_i, bias_f, state, q_start, q_len, slots, o_raw)
     for t, name in ((q_start, "q_start"), (q_len, "q_len"), (slots, "slots")):
@@ -551,9 +551,9 @@ def mlstm_scan(proj: torch.Tensor, bias_i: torch.Tensor, bias_f: torch.Tensor, c
           "mlstm_scan: o_raw is float32 [tokens, heads dv]; key size up to 1,024")
     _need(q_start.numel() == q_len.numel() == slots.numel(), "mlstm_scan: one start, length and slot an entry")
     fn = _fn("mlstm", "kipp_mlstm_scan", [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_size, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
-                                          _c_int, _c_int, _c_int, _c_int, _c_ptr])
+                                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(proj), proj.shape[1], _ptr(bias_i), _ptr(bias_f), float(cap), _ptr(state), state.shape[1], _ptr(q_start),
-              _ptr(q_len), _ptr(slots), _ptr(o_raw), q_start.numel(), heads, d, dv, _stream()), "mlstm_scan")
+              _ptr(q_len), _ptr(slots), _ptr(o_raw), q_start.numel(), heads, d, dv, int(bool(few)), _stream()), "mlstm_scan")
     return o_raw
 
 

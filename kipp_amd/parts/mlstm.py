@@ -81,7 +81,7 @@ class MLSTM:
         proj = rt.linear(x, self.w_in)                    # float32 [n, q | k | v | gate | zi | zf]
         o_raw = rt.empty((n, hv), torch.float32)
         ops.mlstm_scan(proj, self.bias_i, self.bias_f, s.gate_cap, state, batch.q_start, batch.q_len, batch.slots, o_raw,
-                       s.num_heads, s.head_dim, s.v_head_dim)
+                       s.num_heads, s.head_dim, s.v_head_dim, few=batch.max_q_len <= 4)
         out = ops.mlstm_finish(o_raw, proj, 2 * s.num_heads * s.head_dim + hv, self.norm, s.norm_eps, rt.empty((n, hv), rt.act_dtype),
                                s.num_heads, s.v_head_dim)
         return rt.linear(out, self.w_o, slabs=True, defer=True)

@@ -308,6 +308,32 @@ def test_mlstm_scan_and_finish(heads, d, dv):
     assert (state[[1, 3, 5]] == 0).all() and (state[:, size:] == 0).all()      # nothing outside the entries' slots
 
 
+def test_mlstm_scan_for_few_tokens_gives_the_same_bits():
+    """Single tokens take a build with fewer, larger workgroups: the same state and the same output, bit for bit."""
+    import torch
+    from kipp_amd.csrc import ops
+    heads, d, dv = 3, 128, 80
+    rng = np.random.default_rng(4)
+    size = ops.mlstm_state_size(heads, d, dv)
+    proj = dev(rng.normal(size=(6, 2 * heads * d + 2 * heads * dv + 2 * heads)).astype(np.float32))
+    start = torch.tensor(rng.normal(size=(4, size)).astype(np.float32), device="cuda:0")
+    copies = -(-dv // ops.mlstm_columns(d))
+    n0 = start[:, heads * d * dv:heads * d * dv + heads * d].clone()
+    for c in range(copies):         # the copies of n and m of a slot hold the same numbers
+        start[:, heads * d * dv + c * heads * d:heads * d * dv + (c + 1) * heads * d] = n0
+        start[:, heads * d * dv + copies * heads * d + c * heads:heads * d * dv + copies * heads * d + (c + 1) * heads] = start[:, -heads - 4:-4].abs()
+    outs = []
+    for few in (False, True):
+        state = start.clone()
+        o = torch.empty((6, heads * dv), device="cuda:0")
+        for step in range(2):
+            rows = proj[3 * step:3 * step + 3].contiguous()
+            ops.mlstm_scan(rows, dev(np.zeros(heads, np.float32)), dev(np.ones(heads, np.float32)), 7.0, state, dev([0, 1, 2], torch.int32),
+                           dev([1, 1, 1], torch.int32), dev([2, 0, 3], torch.int32), o[3 * step:3 * step + 3], heads, d, dv, few=few)
+        outs.append((o.cpu().numpy(), state.cpu().numpy()))
+    assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1])
+
+
 # =============================================================================== the engine
 
 def requests_of(vocab, seed=0, lengths=LENGTHS):
