@@ -139,7 +139,7 @@ class Attention:
             rt.ops.attention_decode_fused(qkv, cache.k, cache.v, out, batch.decode_rows, batch.positions,
                                           batch.seq_of_token, table, s.num_heads, s.num_kv_heads, s.head_dim,
                                           self.q_norm, self.k_norm, eps, inv_freq, rotary_dim, cache.writable,
-                                          self.scale, s.window or 0, batch.max_decode_ctx, decode_workspace(rt, batch, s.num_heads, s.head_dim),
+                                          self.scale, s.window or 0, batch.max_decode_ctx, self._workspace(batch),
                                           angles=angles, out_steps_major=major)
             return rt.linear(out, self.w_o, slabs=True, defer=True, x_steps_major=major)
         q = rt.ops.qk_norm_rope_kv_write(
@@ -148,8 +148,16 @@ class Attention:
             self.q_norm, self.k_norm, eps, inv_freq, rotary_dim, write_kv=cache.writable, angles=angles, pairing=pairing)
         out = rt.empty((n, s.q_dim), rt.act_dtype)
         paged_attention(rt, batch, q, out, cache.k, cache.v, cache.page_size, table, s.num_heads, s.num_kv_heads, s.head_dim,
-                        s.head_dim, self.scale, s.window, fast)
+                        s.head_dim, self.scale, s.window, fast, owner=self)
         return rt.linear(out, self.w_o, slabs=True, defer=True)
+
+    def _prefill_work(self, batch):
+        """The prefill kernel's work list for this mixer's sizes (`prefill_work`)."""
+        return prefill_work(self.rt, batch, self.spec.num_heads, self.spec.head_dim, self.spec.window)
+
+    def _workspace(self, batch):
+        """The split decode kernel's partial results for this mixer's sizes (`decode_workspace`)."""
+        return decode_workspace(self.rt, batch, self.spec.num_heads, self.spec.head_dim)
 
     def _forward_prepared(self, x, batch, cache):
         """The mixer without rotation and with any of: biases, a norm without weights, a factor on the queries that grows
@@ -177,24 +185,26 @@ class Attention:
             rt.generic_attention_launches += 1
         out = rt.empty((n, s.out_dim), rt.act_dtype)
         paged_attention(rt, batch, q, out, cache.k, cache.v, cache.page_size, table, s.num_heads, s.num_kv_heads, d, dv,
-                        self.scale, s.window, fast)
+                        self.scale, s.window, fast, owner=self)
         return rt.linear(out, self.w_o, slabs=True, defer=True)
 
 
-def paged_attention(rt, batch, q, out, k_cache, v_cache, page_size, table, n_q, n_kv, d, dv, scale, window, fast):
+def paged_attention(rt, batch, q, out, k_cache, v_cache, page_size, table, n_q, n_kv, d, dv, scale, window, fast, owner=None):
     """The attention itself over a paged cache, for any mixer that has its queries ready: q [tokens, n_q d] -> out
     [tokens, n_q dv].  `fast`: the matrix-core kernels (prompt portions and single tokens each by their own; they
     need d == dv, or `v_cache` being `k_cache`, a value then being as wide as its key's row); else the generic kernel,
     which takes values of their own width (`v_cache` may be `k_cache` there too: a value is the first dv numbers
-    of its key's row)."""
+    of its key's row).  `owner`: a mixer whose `_prefill_work(batch)` and `_workspace(batch)` make the work list and the
+    decode workspace (else they are made here for these sizes)."""
     if fast:
         if batch.n_portions:
-            item_seq, item_tile, cuts = prefill_work(rt, batch, n_q, d, window)
+            item_seq, item_tile, cuts = owner._prefill_work(batch) if owner is not None else prefill_work(rt, batch, n_q, d, window)
             rt.ops.attention_prefill(q, k_cache, v_cache, out, item_seq, item_tile, batch.q_start, batch.q_len, batch.positions,
                                      table, n_q, n_kv, d, scale, window or 0, cuts=cuts)
         if batch.n_decode:
             rt.ops.attention_decode(q, k_cache, v_cache, out, batch.decode_rows, batch.positions, batch.seq_of_token, table,
-                                    n_q, n_kv, d, scale, window or 0, batch.max_decode_ctx, decode_workspace(rt, batch, n_q, d))
+                                    n_q, n_kv, d, scale, window or 0, batch.max_decode_ctx,
+                                    owner._workspace(batch) if owner is not None else decode_workspace(rt, batch, n_q, d))
     elif d == dv and v_cache is not k_cache and d <= 256:
         # the float32 path, and geometries the matrix-core kernels refuse (groups above 16, odd page sizes)
         rt.ops.paged_attention_generic(q, k_cache, v_cache, out, batch.positions, batch.seq_of_token, table, n_q, n_kv, d,
