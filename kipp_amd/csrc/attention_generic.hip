@@ -17,6 +17,41 @@
 #define HEADS_PER_BLOCK 4
 #define MAX_D 1024
 
+// q . k over d numbers, added in index order whatever the width of the loads (16 bytes where the row allows).
+__device__ __forceinline__ float dot_row(const float* q, const float* k, int d) {
+    float dot = 0.0f;
+    int e = 0;
+    if ((((uintptr_t)k) & 15) == 0)
+#pragma unroll 4
+        for (; e + 4 <= d; e += 4) {
+            const float4 v = *reinterpret_cast<const float4*>(k + e);
+            dot += q[e] * v.x;
+            dot += q[e + 1] * v.y;
+            dot += q[e + 2] * v.z;
+            dot += q[e + 3] * v.w;
+        }
+    for (; e < d; ++e) dot += q[e] * k[e];
+    return dot;
+}
+
+__device__ __forceinline__ float dot_row(const float* q, const bf16_t* k, int d) {
+    float dot = 0.0f;
+    int e = 0;
+    if ((((uintptr_t)k) & 15) == 0)
+#pragma unroll 4
+        for (; e + 8 <= d; e += 8) {
+            const uint4 v = *reinterpret_cast<const uint4*>(k + e);
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                dot += q[e + 2 * i] * __uint_as_float(w[i] << 16);
+                dot += q[e + 2 * i + 1] * __uint_as_float(w[i] & 0xffff0000u);
+            }
+        }
+    for (; e < d; ++e) dot += q[e] * bf16_to_f32(k[e]);
+    return dot;
+}
+
 template <typename TQ, typename TC, typename TO>
 __global__ void paged_attention_generic_kernel(
     const TQ* __restrict__ q, const TC* __restrict__ k_cache, const TC* __restrict__ v_cache, TO* __restrict__ out,
@@ -56,9 +91,7 @@ __global__ void paged_attention_generic_kernel(
             const int page_id = table[s / page];
             off = ((unsigned long long)page_id * n_kv + g) * page + s % page;
             const TC* k_row = k_cache + off * d;
-            float dot = 0.0f;
-            for (int e = 0; e < d; ++e) dot += q_s[wave][e] * load_f(k_row, e);
-            score = dot * scale;
+            score = dot_row(q_s[wave], k_row, d) * scale;
         }
         const float m_new = fmaxf(m, wave_max(score));
         const float alpha = expf(m - m_new);
@@ -71,13 +104,18 @@ __global__ void paged_attention_generic_kernel(
         __syncthreads();
         const int j_lo = max(0, lo - s0);
         const int j_hi = min(KIPP_WAVE, pos - s0 + 1);
+        // every column's sum still runs over the keys in order; the keys are the outer loop so that a key's loads (one a
+        // column of this lane) and those of the next keys are on their way together
 #pragma unroll
-        for (int c = 0; c < MAX_D / KIPP_WAVE; ++c) {
-            const int e = lane + c * KIPP_WAVE;
-            if (e < dv) {
-                float a = acc[c] * alpha;
-                for (int j = j_lo; j < j_hi; ++j) a += p_s[wave][j] * load_f(v_cache + off_s[wave][j] * v_row, e);
-                acc[c] = a;
+        for (int c = 0; c < MAX_D / KIPP_WAVE; ++c) acc[c] *= alpha;
+#pragma unroll 4
+        for (int j = j_lo; j < j_hi; ++j) {
+            const float pj = p_s[wave][j];
+            const TC* v_at = v_cache + off_s[wave][j] * v_row;
+#pragma unroll
+            for (int c = 0; c < MAX_D / KIPP_WAVE; ++c) {
+                const int e = lane + c * KIPP_WAVE;
+                if (e < dv) acc[c] += pj * load_f(v_at, e);
             }
         }
     }

@@ -20,8 +20,9 @@
 //         lane also keeps its rows of n (the same arithmetic in every column, hence the same bits), so the
 //         denominator needs no exchange between columns either.  The tokens come in chunks: while one chunk is
 //         walked out of LDS, the next one's k, q, v and gate pre-activations are on their way from memory into
-//         registers; tanh, logarithm and the first exponential of the gates are taken once a token by one lane when
-//         the chunk is put into LDS, so the walk itself is multiply-adds, one maximum and three exponentials a token.
+//         registers; when a chunk is put into LDS the first wave takes the gates of its tokens (tanh and logarithms a lane a
+//         token, the running maximum in token order, the exponentials a lane a token again), so the walk itself is
+//         multiply-adds.
 //         The order of a token's operations does not depend on where its chunk begins: a position's bits are the
 //         same however the prompt was cut.
 // finish  every head of a token divided by its root mean square, times the norm's weight, times sigmoid(gate),
@@ -40,7 +41,7 @@ __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.0f) - 
 
 // ROWS rows of a column a lane (a multiple of 4), PARTS lanes a column (side by side in a wave), 256 / PARTS columns a
 // workgroup.  `unit`: columns that share one copy of n and m in the state (a workgroup's columns are a multiple of it).
-// LDS: chunk * (2 ROWS PARTS + columns + 2) floats; rows of k and q are padded with zeros to ROWS * PARTS numbers.
+// LDS: chunk * (2 ROWS PARTS + columns + 4) + 4 floats; rows of k and q are padded with zeros to ROWS * PARTS numbers.
 template <int ROWS, int PARTS>
 __global__ void __launch_bounds__(SCAN_THREADS) mlstm_scan_kernel(
     const float* __restrict__ proj, int stride, const float* __restrict__ bias_i, const float* __restrict__ bias_f, float cap,
@@ -54,8 +55,8 @@ __global__ void __launch_bounds__(SCAN_THREADS) mlstm_scan_kernel(
     float* k_s = lds;
     float* q_s = k_s + (size_t)chunk * DP;
     float* v_s = q_s + (size_t)chunk * DP;
-    float* li_s = v_s + (size_t)chunk * COLS;
-    float* lf_s = li_s + chunk;
+    float* g_s = v_s + (size_t)chunk * COLS;              // a token's (keep, take, floor of the denominator, -)
+    float* m_s = g_s + (size_t)chunk * 4;                  // m after the chunk
     const int seq = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
     const int part = tid & (PARTS - 1), col_l = tid / PARTS;
     const int col = blockIdx.z * COLS + col_l;
@@ -140,9 +141,26 @@ __global__ void __launch_bounds__(SCAN_THREADS) mlstm_scan_kernel(
             const int i = tid + j * SCAN_THREADS;
             if (i < n_tok * COLS) v_s[i] = v_r[j];
         }
-        if (tid < n_tok) {      // the gates' logarithms, a lane a token; the walk below only takes maxima and exponentials
-            li_s[tid] = cap * tanhf((zi + bi) / cap);
-            lf_s[tid] = log_sigmoid(cap * tanhf((zf + bf) / cap));
+        if (tid < KIPP_WAVE) {
+            // The gates, by the first wave: a lane a token takes tanh and the logarithms; then the running maximum walks the
+            // chunk's tokens in order (m' = max(lf + m, li): an add and a maximum a token, the lanes' numbers read across
+            // the wave), and every lane takes its token's three exponentials.  The walk below is left with multiply-adds.
+            const float li = tid < n_tok ? cap * tanhf((zi + bi) / cap) : 0.0f;
+            const float lf = tid < n_tok ? log_sigmoid(cap * tanhf((zf + bf) / cap)) : 0.0f;
+            float m_before = 0.0f, m_after = 0.0f;
+            for (int t = 0; t < n_tok; ++t) {
+                const float lf_t = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(lf), t));
+                const float li_t = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(li), t));
+                const float m_new = fmaxf(lf_t + m, li_t);
+                if (tid == t) {
+                    m_before = m;
+                    m_after = m_new;
+                }
+                m = m_new;
+            }
+            if (tid < n_tok)
+                *reinterpret_cast<float4*>(g_s + 4 * tid) = make_float4(expf(lf + m_before - m_after), expf(li - m_after), expf(-m_after), 0.0f);
+            if (tid == 0) m_s[0] = m;
         }
         __syncthreads();
         const int n_next = min(chunk, count - c0 - chunk);
@@ -154,13 +172,10 @@ __global__ void __launch_bounds__(SCAN_THREADS) mlstm_scan_kernel(
             float keep[SCAN_GROUP], take[SCAN_GROUP], floor_p[SCAN_GROUP], num_p[SCAN_GROUP], den_p[SCAN_GROUP];
 #pragma unroll
             for (int u = 0; u < SCAN_GROUP; ++u) {
-                const int tt = min(t8 + u, n_tok - 1);
-                const float li = li_s[tt], lf = lf_s[tt];
-                const float m_new = t8 + u < n_tok ? fmaxf(lf + m, li) : m;
-                keep[u] = expf(lf + m - m_new);
-                take[u] = expf(li - m_new);
-                floor_p[u] = expf(-m_new);
-                m = m_new;
+                const float4 g = *reinterpret_cast<const float4*>(g_s + 4 * min(t8 + u, n_tok - 1));
+                keep[u] = g.x;
+                take[u] = g.y;
+                floor_p[u] = g.z;
             }
 #pragma unroll
             for (int u = 0; u < SCAN_GROUP; ++u) {
@@ -224,7 +239,7 @@ __global__ void __launch_bounds__(SCAN_THREADS) mlstm_scan_kernel(
             if (writes_copy && row < d) n_w[row] = nv[r];
         }
     }
-    if (writes_copy && part == 0) m_all[(size_t)(col / unit) * heads + head] = m;
+    if (writes_copy && part == 0) m_all[(size_t)(col / unit) * heads + head] = m_s[0];
 }
 
 #define FINISH_HEADS 4
@@ -268,7 +283,7 @@ int kipp_mlstm_scan(const float* proj, int stride, const float* bias_i, const fl
     dim3 grid(n_seqs, heads, (dv + cols - 1) / cols), block(SCAN_THREADS);
     int chunk = SCAN_STAGE / (rows * parts);          // tokens whose k and q fit the staging registers
     if (chunk > 32) chunk = 32;
-    const size_t lds = (size_t)chunk * (2 * rows * parts + cols + 2) * sizeof(float);
+    const size_t lds = ((size_t)chunk * (2 * rows * parts + cols + 4) + 4) * sizeof(float);
 #define KIPP_SCAN(R, P)                                                                                                          \
     hipLaunchKernelGGL((mlstm_scan_kernel<R, P>), grid, block, lds, stream, proj, stride, bias_i, bias_f, cap, state, state_stride, \
                        q_start, q_len, slots, o_raw, heads, d, dv, chunk, unit, copies)
