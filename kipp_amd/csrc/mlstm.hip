@@ -40,9 +40,10 @@
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.0f) - log1pf(expf(-fabsf(z))); }
 
 // ROWS rows of a column a lane (a multiple of 4), PARTS lanes a column (side by side in a wave), 256 / PARTS columns a
-// workgroup.  `unit`: columns that share one copy of n and m in the state (a workgroup's columns are a multiple of it).
+// workgroup.  BASE: the rows a lane has in the build for prompt portions of this key size; a build with more rows a lane
+// adds them in runs of BASE and the runs pairwise, which is the order in which the lanes of that build add theirs.  `unit`: columns that share one copy of n and m in the state (a workgroup's columns are a multiple of it).
 // LDS: chunk * (2 ROWS PARTS + columns + 4) + 4 floats; rows of k and q are padded with zeros to ROWS * PARTS numbers.
-template <int ROWS, int PARTS>
+template <int ROWS, int PARTS, int BASE>
 __global__ void __launch_bounds__(SCAN_THREADS) mlstm_scan_kernel(
     const float* __restrict__ proj, int stride, const float* __restrict__ bias_i, const float* __restrict__ bias_f, float cap,
     float* __restrict__ state, size_t state_stride, const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
@@ -191,9 +192,8 @@ __global__ void __launch_bounds__(SCAN_THREADS) mlstm_scan_kernel(
                         *reinterpret_cast<float4*>(kk + r) = *reinterpret_cast<const float4*>(k_t + r);
                         *reinterpret_cast<float4*>(qq + r) = *reinterpret_cast<const float4*>(q_t + r);
                     }
-                    // rows are summed in runs of 8 and the runs pairwise, as the lanes of the 8-row build add theirs:
-                    // the build with 32 rows a lane (few tokens an entry) gives the same bits
-                    constexpr int RUNS = ROWS == 32 ? 4 : 1;
+                    constexpr int RUNS = ROWS / BASE;
+                    static_assert(RUNS == 1 || RUNS == 2 || RUNS == 4, "runs of rows");
                     float num[RUNS], den[RUNS];
 #pragma unroll
                     for (int g = 0; g < RUNS; ++g) num[g] = den[g] = 0.0f;
@@ -201,11 +201,11 @@ __global__ void __launch_bounds__(SCAN_THREADS) mlstm_scan_kernel(
                     for (int r = 0; r < ROWS; ++r) {
                         S[r] = fmaf(keep[u], S[r], kk[r] * tv);
                         nv[r] = fmaf(keep[u], nv[r], take[u] * kk[r]);
-                        num[r / (ROWS / RUNS)] = fmaf(S[r], qq[r], num[r / (ROWS / RUNS)]);
-                        den[r / (ROWS / RUNS)] = fmaf(nv[r], qq[r], den[r / (ROWS / RUNS)]);
+                        num[r / BASE] = fmaf(S[r], qq[r], num[r / BASE]);
+                        den[r / BASE] = fmaf(nv[r], qq[r], den[r / BASE]);
                     }
-                    num_p[u] = RUNS == 4 ? (num[0] + num[1]) + (num[RUNS / 2] + num[RUNS - 1]) : num[0];
-                    den_p[u] = RUNS == 4 ? (den[0] + den[1]) + (den[RUNS / 2] + den[RUNS - 1]) : den[0];
+                    num_p[u] = RUNS == 4 ? (num[0] + num[1]) + (num[RUNS / 2] + num[RUNS - 1]) : (RUNS == 2 ? num[0] + num[RUNS - 1] : num[0]);
+                    den_p[u] = RUNS == 4 ? (den[0] + den[1]) + (den[RUNS / 2] + den[RUNS - 1]) : (RUNS == 2 ? den[0] + den[RUNS - 1] : den[0]);
                 }
             }
 #pragma unroll
@@ -261,9 +261,9 @@ __global__ void mlstm_finish_kernel(const float* __restrict__ o_raw, const float
         store_f(dst, e, src[e] * scale * norm_w[head * dv + e] * (1.0f / (1.0f + expf(-gate[e]))));
 }
 
-// Lanes that share a column of the memory in the walk over prompt portions: 8 rows a lane (16 for keys of more than
-// 512 numbers).  256 / lanes is the `unit`: the columns that share a copy of n and m in the state.
-static int kipp_mlstm_parts(int d) { return d <= 32 ? 4 : (d <= 128 ? 16 : 64); }
+// Lanes that share a column of the memory in the walk over prompt portions: 8 rows a lane (16 for keys of 129 to 256 and
+// of more than 512 numbers).  256 / lanes is the `unit`: the columns that share a copy of n and m in the state.
+static int kipp_mlstm_parts(int d) { return d <= 32 ? 4 : (d <= 256 ? 16 : 64); }
 
 extern "C" {
 
@@ -277,21 +277,26 @@ int kipp_mlstm_scan(const float* proj, int stride, const float* bias_i, const fl
     const int unit = SCAN_THREADS / kipp_mlstm_parts(d);
     const int copies = (dv + unit - 1) / unit;
     if (stride < 2 * heads * d + 2 * heads * dv + 2 * heads || state_stride < (size_t)heads * d * dv + (size_t)copies * (heads * d + heads)) return -1;
-    const int parts = (few && d > 32 && d <= 128) ? 4 : kipp_mlstm_parts(d);
-    const int rows = parts == 4 ? (d <= 32 ? 8 : 32) : (d <= 512 ? 8 : 16);
+    const int base_parts = kipp_mlstm_parts(d);
+    const int base_rows = d <= 128 ? 8 : (d <= 256 ? 16 : (d <= 512 ? 8 : 16));
+    int parts = base_parts, rows = base_rows;
+    if (few && d > 32 && d <= 128) parts = 4, rows = 32;
+    else if (few && d > 128 && d <= 256) parts = 8, rows = 32;
     const int cols = SCAN_THREADS / parts;
     dim3 grid(n_seqs, heads, (dv + cols - 1) / cols), block(SCAN_THREADS);
     int chunk = SCAN_STAGE / (rows * parts);          // tokens whose k and q fit the staging registers
     if (chunk > 32) chunk = 32;
     const size_t lds = ((size_t)chunk * (2 * rows * parts + cols + 4) + 4) * sizeof(float);
-#define KIPP_SCAN(R, P)                                                                                                          \
-    hipLaunchKernelGGL((mlstm_scan_kernel<R, P>), grid, block, lds, stream, proj, stride, bias_i, bias_f, cap, state, state_stride, \
+#define KIPP_SCAN(R, P, B)                                                                                                          \
+    hipLaunchKernelGGL((mlstm_scan_kernel<R, P, B>), grid, block, lds, stream, proj, stride, bias_i, bias_f, cap, state, state_stride, \
                        q_start, q_len, slots, o_raw, heads, d, dv, chunk, unit, copies)
-    if (parts == 4 && rows == 8) KIPP_SCAN(8, 4);
-    else if (parts == 4) KIPP_SCAN(32, 4);
-    else if (parts == 16) KIPP_SCAN(8, 16);
-    else if (rows == 8) KIPP_SCAN(8, 64);
-    else KIPP_SCAN(16, 64);
+    if (parts == 4 && rows == 8) KIPP_SCAN(8, 4, 8);
+    else if (parts == 4) KIPP_SCAN(32, 4, 8);
+    else if (parts == 8) KIPP_SCAN(32, 8, 16);
+    else if (parts == 16 && rows == 8) KIPP_SCAN(8, 16, 8);
+    else if (parts == 16) KIPP_SCAN(16, 16, 16);
+    else if (rows == 8) KIPP_SCAN(8, 64, 8);
+    else KIPP_SCAN(16, 64, 16);
 #undef KIPP_SCAN
     return KIPP_LAUNCH_CHECK();
 }

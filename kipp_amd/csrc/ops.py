@@ -523,7 +523,7 @@ def latent_expand(lat: torch.Tensor, w_uv_t: torch.Tensor, out: torch.Tensor, he
 
 def mlstm_columns(d: int) -> int:
     """Columns of the memory that a workgroup of the scan takes (fewer where a column's rows need more lanes)."""
-    return 256 // (4 if d <= 32 else (16 if d <= 128 else 64))
+    return 256 // (4 if d <= 32 else (16 if d <= 256 else 64))
 
 
 def mlstm_state_size(heads: int, d: int, dv: int) -> int:

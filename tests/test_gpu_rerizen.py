@@ -308,11 +308,11 @@ def test_mlstm_scan_and_finish(heads, d, dv):
     assert (state[[1, 3, 5]] == 0).all() and (state[:, size:] == 0).all()      # nothing outside the entries' slots
 
 
-def test_mlstm_scan_for_few_tokens_gives_the_same_bits():
+@pytest.mark.parametrize("heads, d, dv", [(3, 128, 80), (2, 200, 40), (2, 256, 72), (2, 24, 70)])
+def test_mlstm_scan_for_few_tokens_gives_the_same_bits(heads, d, dv):
     """Single tokens take a build with fewer, larger workgroups: the same state and the same output, bit for bit."""
     import torch
     from kipp_amd.csrc import ops
-    heads, d, dv = 3, 128, 80
     rng = np.random.default_rng(4)
     size = ops.mlstm_state_size(heads, d, dv)
     proj = dev(rng.normal(size=(6, 2 * heads * d + 2 * heads * dv + 2 * heads)).astype(np.float32))
