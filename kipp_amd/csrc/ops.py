@@ -348,22 +348,31 @@ def _streams_write_args(x, delta, mix, outw, what):
 
 
 def streams_step(x: torch.Tensor, delta: Optional[torch.Tensor], mix: Optional[torch.Tensor], outw: Optional[torch.Tensor],
-                 inw: Optional[torch.Tensor], norm_w: Optional[torch.Tensor], eps: float, h: Optional[torch.Tensor]):
+                 inw: Optional[torch.Tensor], norm_w: Optional[torch.Tensor], eps: float, h: Optional[torch.Tensor],
+                 which: Optional[torch.Tensor] = None, store: bool = True):
     """One pass over the R rows of every token of x [tokens, R, width] (float32): with `delta` (a sublayer's result,
     maybe in slabs) the rows become X_t <- sum_r mix[r, t] X_r + outw[t] delta; with `inw` the weighted sum
-    sum_r inw[r] X_r is RMS-normed with `norm_w` into `h` [tokens, width]."""
+    sum_r inw[r] X_r is RMS-normed with `norm_w` into `h` [tokens, width].  `which` (int32 token numbers) with `store`
+    False: only those tokens are read, into `h` [len(which), width], and the written rows are not stored (the last read
+    of a forward pass, when only some rows go on)."""
     _dev(x, delta, mix, outw, inw, norm_w, h)
     _need(x.dim() == 3 and x.dtype == torch.float32 and 0 < x.shape[1] <= STREAMS_MAX, "streams_step: x is float32 [tokens, R <= 8, width]")
     n, r, width = x.shape
     parts = _streams_write_args(x, delta, mix, outw, "streams_step")
     if inw is not None:
         _need(inw.dtype == torch.float32 and inw.numel() == r and norm_w is not None and norm_w.dtype == torch.float32
-              and norm_w.numel() == width and h is not None and h.shape == (n, width), "streams_step: float32 [R] and [width], h [tokens, width]")
+              and norm_w.numel() == width and h is not None and h.shape == (n if which is None else which.numel(), width),
+              "streams_step: float32 [R] and [width], h [rows, width]")
     _need(delta is not None or inw is not None, "streams_step: nothing to do")
+    if which is not None:
+        _dev(which)
+        _i32(which, "which")
+        _need(not store and inw is not None, "streams_step: named rows are read only, and nothing is stored")
     fn = _fn("streams", "kipp_streams_step", [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_int,
-                                              _c_int, _c_int, _c_int, _c_ptr])
+                                              _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(x), _ptr(delta), parts, _ptr(mix), _ptr(outw), _ptr(inw), _ptr(norm_w), float(eps),
-              _ptr(h) if inw is not None else None, _code(h) if inw is not None else F32, n, r, width, _stream()), "streams_step")
+              _ptr(h) if inw is not None else None, _code(h) if inw is not None else F32, n, r, width, _ptr(which),
+              which.numel() if which is not None else n, int(bool(store)), _stream()), "streams_step")
     return h
 
 

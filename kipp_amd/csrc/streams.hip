@@ -31,20 +31,6 @@ __global__ void streams_open_kernel(const TT* __restrict__ table, const int32_t*
     }
 }
 
-struct StreamCoefficients {
-    float mix[STREAMS_MAX][STREAMS_MAX];   // [from][to]
-    float out[STREAMS_MAX];
-    float in[STREAMS_MAX];
-};
-
-__device__ __forceinline__ void load_coefficients(StreamCoefficients& c, const float* mix, const float* outw, const float* inw, int R) {
-    for (int s = 0; s < R; ++s) {
-        for (int t = 0; t < R; ++t) c.mix[s][t] = mix != nullptr ? mix[s * R + t] : 0.0f;
-        c.out[s] = outw != nullptr ? outw[s] : 0.0f;
-        c.in[s] = inw != nullptr ? inw[s] : 0.0f;
-    }
-}
-
 // write (if mix != nullptr), then read and norm (if inw != nullptr).  R copies (a build constant where it is 1 to 4, so
 // that the coefficients and a lane's rows stay in registers), VEC numbers a lane and load (4 where the width
 // allows); the workgroup is sized so that a lane meets its numbers once where the width allows, with every load
@@ -53,10 +39,10 @@ template <int RMAX, int VEC, typename TO>
 __global__ void streams_step_kernel(float* __restrict__ X, const float* __restrict__ delta, int parts, size_t part_stride,
                                     const float* __restrict__ mix, const float* __restrict__ outw,
                                     const float* __restrict__ inw, const float* __restrict__ norm_w, float eps,
-                                    TO* __restrict__ h, int R, int width) {
+                                    TO* __restrict__ h, int R, int width, const int32_t* __restrict__ which, int store) {
     extern __shared__ float lds[];
     float* u_s = lds + 16;
-    const int t = blockIdx.x;
+    const int t = which != nullptr ? which[blockIdx.x] : blockIdx.x;     // the token; the normed row leaves as row blockIdx.x
     float* rows = X + (size_t)t * R * width;
     float c_mix[RMAX][RMAX], c_out[RMAX], c_in[RMAX];
 #pragma unroll
@@ -99,7 +85,7 @@ __global__ void streams_step_kernel(float* __restrict__ X, const float* __restri
                     for (int s = 0; s < RMAX; ++s) acc += c_mix[s][to] * x[s][v];
                     fresh[to][v] = acc + c_out[to] * y[v];
                 }
-                if (to < R) {
+                if (to < R && store) {
                     if (VEC == 4) *reinterpret_cast<float4*>(rows + (size_t)to * width + e) = *reinterpret_cast<float4*>(fresh[to]);
                     else rows[(size_t)to * width + e] = fresh[to][0];
                 }
@@ -123,42 +109,44 @@ __global__ void streams_step_kernel(float* __restrict__ X, const float* __restri
     if (inw == nullptr) return;
     ss = block_sum(ss, lds);
     const float scale = 1.0f / sqrtf(ss / (float)width + eps);
-    TO* dst = h + (size_t)t * width;
+    TO* dst = h + (size_t)blockIdx.x * width;
     for (int e = threadIdx.x * VEC; e < width; e += blockDim.x * VEC)
 #pragma unroll
         for (int v = 0; v < VEC; ++v) store_f(dst, e + v, u_s[e + v] * scale * norm_w[e + v]);
 }
 
+template <int RMAX>
 __global__ void streams_close_kernel(const float* __restrict__ X, const float* __restrict__ delta, int parts, size_t part_stride,
                                      const float* __restrict__ mix, const float* __restrict__ outw,
                                      const int32_t* __restrict__ which, float* __restrict__ out, int R, int width) {
     const int i = blockIdx.x;
     const int t = which != nullptr ? which[i] : i;
     const float* rows = X + (size_t)t * R * width;
-    StreamCoefficients c;
-    load_coefficients(c, mix, outw, nullptr, R);
-    for (int e = threadIdx.x; e < width; e += blockDim.x) {
-        float x[STREAMS_MAX];
+    float c_mix[RMAX][RMAX], c_out[RMAX];
 #pragma unroll
-        for (int r = 0; r < STREAMS_MAX; ++r) x[r] = r < R ? rows[(size_t)r * width + e] : 0.0f;
+    for (int s = 0; s < RMAX; ++s) {
+#pragma unroll
+        for (int to = 0; to < RMAX; ++to) c_mix[s][to] = (mix != nullptr && s < R && to < R) ? mix[s * R + to] : 0.0f;
+        c_out[s] = (outw != nullptr && s < R) ? outw[s] : 0.0f;
+    }
+    for (int e = threadIdx.x; e < width; e += blockDim.x) {
+        float x[RMAX];
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r) x[r] = r < R ? rows[(size_t)r * width + e] : 0.0f;
         float total = 0.0f;
         if (mix != nullptr) {
             float y = 0.0f;
             for (int p = 0; p < parts; ++p) y += delta[p * part_stride + (size_t)t * width + e];
 #pragma unroll
-            for (int to = 0; to < STREAMS_MAX; ++to) {
-                if (to < R) {
-                    float v = 0.0f;
+            for (int to = 0; to < RMAX; ++to) {
+                float v = 0.0f;
 #pragma unroll
-                    for (int s = 0; s < STREAMS_MAX; ++s)
-                        if (s < R) v += c.mix[s][to] * x[s];
-                    total += v + c.out[to] * y;
-                }
+                for (int s = 0; s < RMAX; ++s) v += c_mix[s][to] * x[s];
+                if (to < R) total += v + c_out[to] * y;
             }
         } else {
 #pragma unroll
-            for (int r = 0; r < STREAMS_MAX; ++r)
-                if (r < R) total += x[r];
+            for (int r = 0; r < RMAX; ++r) total += x[r];
         }
         out[(size_t)i * width + e] = total;
     }
@@ -179,10 +167,14 @@ int kipp_streams_open(const void* table, int table_dtype, const int32_t* tokens,
     return KIPP_LAUNCH_CHECK();
 }
 
-// delta/mix/outw null: no write.  inw null: no read (h unused).
+// delta/mix/outw null: no write.  inw null: no read (h unused).  `which` (n_rows token numbers, or null: all n tokens in
+// order): the tokens that are read; `store` 0: the written copies are not stored (the last read of a forward pass).
 int kipp_streams_step(float* X, const float* delta, int parts, const float* mix, const float* outw, const float* inw,
-                      const float* norm_w, float eps, void* h, int h_dtype, int n, int R, int width, hipStream_t stream) {
-    if (n <= 0) return 0;
+                      const float* norm_w, float eps, void* h, int h_dtype, int n, int R, int width, const int32_t* which,
+                      int n_rows, int store, hipStream_t stream) {
+    if (which == nullptr) n_rows = n;
+    if (n <= 0 || n_rows <= 0) return 0;
+    if (which != nullptr && store) return -2;
     if (R <= 0 || R > STREAMS_MAX || width <= 0 || width > 32768) return -1;
     if ((mix == nullptr) != (delta == nullptr) || (mix != nullptr && outw == nullptr)) return -2;
     if (inw != nullptr && (norm_w == nullptr || h == nullptr)) return -2;
@@ -192,8 +184,8 @@ int kipp_streams_step(float* X, const float* delta, int parts, const float* mix,
     const int lanes = wide ? width / 4 : width;
     const int threads = lanes >= 1024 ? 1024 : ((lanes + KIPP_WAVE - 1) / KIPP_WAVE) * KIPP_WAVE;
 #define KIPP_SS(RMAX, VEC, TO)                                                                                                  \
-    hipLaunchKernelGGL((streams_step_kernel<RMAX, VEC, TO>), dim3(n), dim3(threads), lds, stream, X, delta, parts, stride, mix, \
-                       outw, inw, norm_w, eps, (TO*)h, R, width)
+    hipLaunchKernelGGL((streams_step_kernel<RMAX, VEC, TO>), dim3(n_rows), dim3(threads), lds, stream, X, delta, parts, stride, mix, \
+                       outw, inw, norm_w, eps, (TO*)h, R, width, which, store)
 #define KIPP_SS_R(VEC, TO)                   \
     do {                                     \
         if (R == 1) KIPP_SS(1, VEC, TO);     \
@@ -217,8 +209,13 @@ int kipp_streams_close(const float* X, const float* delta, int parts, const floa
     if (n_out <= 0) return 0;
     if (R <= 0 || R > STREAMS_MAX || width <= 0) return -1;
     if ((mix == nullptr) != (delta == nullptr) || (mix != nullptr && outw == nullptr)) return -2;
-    hipLaunchKernelGGL(streams_close_kernel, dim3(n_out), dim3(block_for(width)), 0, stream, X, delta, parts, (size_t)n * width, mix,
-                       outw, which, out, R, width);
+#define KIPP_SC(RMAX)                                                                                                     \
+    hipLaunchKernelGGL(streams_close_kernel<RMAX>, dim3(n_out), dim3(block_for(width)), 0, stream, X, delta, parts,           \
+                       (size_t)n * width, mix, outw, which, out, R, width)
+    if (R <= 2) KIPP_SC(2);
+    else if (R <= 4) KIPP_SC(4);
+    else KIPP_SC(STREAMS_MAX);
+#undef KIPP_SC
     return KIPP_LAUNCH_CHECK();
 }
 

@@ -139,7 +139,7 @@ class Model:
 def _forward_streams(self, batch, cache) -> Optional[torch.Tensor]:
     """The forward pass of a model that keeps several copies of the residual stream: x is [tokens, R, width], every
     copy the token's embedding at the start; the blocks read and write the copies; the final norm reads their sum."""
-    from ..parts.streams import close_streams, open_streams
+    from ..parts.streams import close_norm_streams, open_streams
     if self.input_position is not None or float(getattr(self.spec.embedding, "scale", 1.0)) != 1.0:
         raise NotImplementedError("several residual streams with a scaled embedding or a position part on the stream")
     x = open_streams(self.rt, self.embedding.weight, batch.tokens, self.spec.streams)
@@ -150,8 +150,9 @@ def _forward_streams(self, batch, cache) -> Optional[torch.Tensor]:
     if batch.n_want == 0:
         # nothing is asked for, and the last write has no reader: the step's work for the caches and states is done
         return None
-    rows = close_streams(self.rt, x, pending, None if batch.want_every_row else batch.want_rows)
-    return self.head.forward(self.final_norm.forward(rows, self.rt.act_dtype))
+    if not hasattr(self.final_norm, "weight") or not hasattr(self.final_norm.spec, "eps"):
+        raise NotImplementedError("several residual streams end in an RMS norm")
+    return self.head.forward(close_norm_streams(self.rt, x, pending, None if batch.want_every_row else batch.want_rows, self.final_norm))
 
 
 Model._forward_streams = _forward_streams

@@ -112,6 +112,20 @@ def open_streams(rt, table, tokens, streams: int):
     return rt.ops.streams_open(table, tokens, rt.empty((tokens.numel(), streams, table.shape[1]), torch.float32))
 
 
+def close_norm_streams(rt, x, pending, which, norm):
+    """[rows, width] in the type the products read: the last write carried out without being stored, the sum of the copies
+    RMS-normed by `norm` (the final norm), for the rows `which` names (None: every token in order).  One kernel."""
+    ones = getattr(rt, "_stream_ones", None)
+    if ones is None or ones.numel() < x.shape[1]:
+        ones = rt._stream_ones = torch.ones(8, dtype=torch.float32, device=rt.device)
+    rows = x.shape[0] if which is None else which.numel()
+    h = rt.empty((rows, x.shape[2]), rt.act_dtype)
+    if pending is None:
+        return rt.ops.streams_step(x, None, None, None, ones[:x.shape[1]], norm.weight, norm.spec.eps, h, which=which, store=False)
+    return rt.ops.streams_step(x, rt.settle(pending.delta), pending.connection.mix, pending.connection.out, ones[:x.shape[1]],
+                               norm.weight, norm.spec.eps, h, which=which, store=False)
+
+
 def close_streams(rt, x, pending, which):
     """float32 [rows, width]: the sum of the copies after the last write (not stored), for the rows `which` names
     (None: every token in order)."""

@@ -95,6 +95,11 @@ def test_streams_kernels(R, width):
     which = [4, 1]
     s = ops.streams_close(dev(x0), dev(delta), dev(mix), dev(outw), dev(which, torch.int32), torch.empty((2, width), device="cuda:0"))
     assert np.allclose(s.cpu().numpy(), ref_x.sum(0)[which], rtol=3e-5, atol=3e-5)
+    # the last read of a forward pass: named rows, the write carried out but not stored, the sum of the copies normed
+    X3 = dev(x0)
+    h3 = ops.streams_step(X3, dev(delta), dev(mix), dev(outw), dev(np.ones(R, np.float32)), dev(w), 1e-5,
+                          torch.empty((2, width), device="cuda:0"), which=dev(which, torch.int32), store=False)
+    assert np.allclose(h3.cpu().numpy(), P.norm(ref_x.sum(0)[which], w, 1e-5), rtol=3e-5, atol=3e-5) and np.array_equal(X3.cpu().numpy(), x0)
     s = ops.streams_close(dev(x0), None, None, None, None, torch.empty((n, width), device="cuda:0"))
     assert np.allclose(s.cpu().numpy(), x0.astype(np.float64).sum(1), rtol=1e-5, atol=1e-5)
 
