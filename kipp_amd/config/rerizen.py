@@ -106,6 +106,11 @@ class RerizenConfig:
             source = _int(m, "kv_from", where, 0)
             if source >= i:
                 raise ConfigError(f"config.json {where}kv_from: layer {source} is not an earlier layer")
+        if source is not None and 0 <= source < len(self.layers) and isinstance(self.layers[source], dict) \
+                and isinstance(self.layers[source].get("mixer"), dict):
+            # a layer that reads another's keys and values may leave their sizes to that layer
+            theirs = self.layers[source]["mixer"]
+            m = dict({k: theirs[k] for k in ("kv_heads", "dim", "vdim") if k in theirs and k not in m}, **m)
         dim, vdim = _int(m, "dim", where), _int(m, "vdim", where)
         spec = AttentionSpec(
             hidden_size=self.width, num_heads=_int(m, "heads", where), num_kv_heads=_int(m, "kv_heads", where), head_dim=dim,

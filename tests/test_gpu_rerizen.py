@@ -170,6 +170,67 @@ def test_head_prepare_and_wide_attention(dtype, H_, G, d, dv, norm, temp):
         assert np.allclose(out.float().cpu().numpy(), want, rtol=tol, atol=tol * np.abs(want).max()), (dtype, queries)
 
 
+def attention_batch(case, T, queries):
+    """What `paged_attention` reads of a step's batch, for one prompt portion of T rows or for single tokens at `queries`."""
+    import types
+
+    import torch
+    from kipp_amd.engine.batch import StepBatch
+
+    class B:
+        pass
+    b = B()
+    b.n_portions, b.n_decode = (1, 0) if queries is None else (0, len(queries))
+    b.q_start = dev([0] if queries is None else list(range(len(queries))), torch.int32)
+    b.q_len = dev([T] if queries is None else [1] * len(queries), torch.int32)
+    b.positions, b.seq_of_token = case.positions, case.seq_of
+    b.decode_rows = dev(list(range(len(queries))) if queries else [0], torch.int32)
+    b.max_decode_ctx = T
+    b.n_tokens = case.rows
+    b.host = {"q_start": [0] if queries is None else list(range(len(queries))), "q_len": [T] if queries is None else [1] * len(queries),
+              "ctx_len": [T] if queries is None else [p_ + 1 for p_ in queries]}
+    b.step_cache = {}
+    b.upload = types.MethodType(StepBatch.upload, b)
+    b.tokens = case.positions
+    return b
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("key", [0, 2, 15, 16, 255, 256])
+def test_a_far_key_takes_the_softmax(dtype, key):
+    """One key among 300, at the sequence's start and on both sides of page and tile borders, points where the last query
+    points after the head norm and the query factor: the last row's result is that key's value, for the row of a prompt
+    portion and for a single token, on the matrix-core kernels and on the generic one."""
+    import torch
+    from kipp_amd.csrc import ops
+    from kipp_amd.parts.mixer import paged_attention
+    from kipp_amd.runtime import Runtime
+    rt = Runtime(dtype)
+    act = rt.act_dtype
+    H_, G, d, dv, T, page, scale = 4, 2, 32, 32, 300, 16, 1.0
+    rng = np.random.default_rng(key)
+    proj = rng.normal(size=(T, H_ * d + G * d + G * dv)).astype(np.float32)
+    u = rng.normal(size=d).astype(np.float32)
+    for h in range(H_):
+        proj[T - 1, h * d:(h + 1) * d] = 5.0 * u             # the norm takes the length away, the direction stays
+    for g in range(G):
+        proj[key, H_ * d + g * d:H_ * d + (g + 1) * d] = -3.0 * u if key == T - 1 else 3.0 * u
+        proj[key, H_ * d + G * d + g * dv:H_ * d + G * d + (g + 1) * dv] = 200.0
+    for fast in ([False, True] if dtype == "bfloat16" else [False]):
+        for queries in (None, [T - 1]):
+            whole, case = PagedCase(T, page, None, seed=1), PagedCase(T, page, queries, seed=1)
+            kc = torch.zeros((case.pages, G, page, d), dtype=act, device="cuda:0")
+            vc = torch.zeros((case.pages, G, page, dv), dtype=act, device="cuda:0")
+            q = ops.head_prepare(dev(proj), torch.empty((T, H_ * d), dtype=act, device="cuda:0"), kc, vc, whole.positions, whole.seq_of,
+                                 whole.table, H_, G, d, dv, None, "plain", 1e-5, None, None, 0.5, 64)
+            if queries is not None:
+                q = q[queries].contiguous()
+            out = torch.zeros((case.rows, H_ * dv), dtype=act, device="cuda:0")
+            paged_attention(rt, attention_batch(case, T, queries), q, out, kc, vc, page, case.table, H_, G, d, dv, scale, None, fast)
+            last = out[-1].float().cpu().numpy()
+            assert np.allclose(last, 200.0, rtol=2e-2), (dtype, fast, queries, last[:4])
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("heads, d, dr, dv, q_rank, rank, rot_dims, window, fast", [
     (4, 32, 16, 24, 64, 48, 16, 40, True), (5, 24, 8, 20, 40, 36, 8, None, False), (2, 16, 12, 48, 24, 20, 8, 7, False),
@@ -244,23 +305,7 @@ def test_latent_kernels_with_a_key_that_stands_out(dtype, heads, d, dr, dv, q_ra
             widthv = row if use_fast else rank
             lat = torch.zeros((case.rows, heads * widthv), dtype=act, device="cuda:0")
 
-            class B:        # what paged_attention reads of a batch
-                pass
-            b = B()
-            import types
-            b.n_portions, b.n_decode = (1, 0) if queries is None else (0, len(queries))
-            b.q_start = dev([0] if queries is None else list(range(len(queries))), torch.int32)
-            b.q_len = dev([T] if queries is None else [1] * len(queries), torch.int32)
-            b.positions, b.seq_of_token = case.positions, case.seq_of
-            b.decode_rows = dev(list(range(len(queries))) if queries else [0], torch.int32)
-            b.max_decode_ctx = T
-            b.n_tokens = case.rows
-            b.host = {"q_start": [0] if queries is None else list(range(len(queries))), "q_len": [T] if queries is None else [1] * len(queries),
-                      "ctx_len": [T] if queries is None else [p_ + 1 for p_ in queries]}
-            b.step_cache = {}
-            from kipp_amd.engine.batch import StepBatch
-            b.upload = types.MethodType(StepBatch.upload, b)
-            b.tokens = case.positions
+            b = attention_batch(case, T, queries)
             paged_attention(rt, b, ql, lat, cache, cache, page, case.table, heads, 1, row, widthv, scale, window, use_fast)
             uv_t = dev(w["uv"].astype(np.float32)).to(act).view(heads, dv, rank).transpose(1, 2).contiguous()
             gate_src = dev(proj) if queries is None else dev(proj[queries])

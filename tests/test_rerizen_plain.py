@@ -191,6 +191,14 @@ def test_configuration_builds_the_model_as_data():
     assert parse_config(typed.to_dict())[1] == typed
 
 
+def test_a_layer_that_reads_anothers_keys_may_leave_their_sizes_out():
+    cfg = shape_config("rerizen-tiny-a")
+    for key in ("kv_heads", "dim", "vdim"):
+        del cfg["layers"][3]["mixer"][key]
+    mixer = parse_config(cfg)[1].model_spec().layers[3].part("mixer")
+    assert (mixer.num_kv_heads, mixer.head_dim, mixer.value_dim, mixer.own_kv) == (2, 32, 32, False)
+
+
 def test_configuration_without_streams_is_one_plain_residual():
     from kipp_amd.engine.model import model_params
     cfg = shape_config("rerizen-tiny-b")
