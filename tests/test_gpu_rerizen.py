@@ -483,6 +483,52 @@ def test_other_sizes_and_branches(tmp_path, dtype):
                 close(got[rid], plain_logits(folder, toks), TOL[dtype] * (4 if dtype == "bfloat16" else 1), f"{width}/{dtype}/{rid}")
 
 
+def random_configuration(rng):
+    """A model of the design with every size, the order of its layers and every constant drawn at random."""
+    layers, sources = [], []
+    for i in range(rng.randint(3, 6)):
+        kind = rng.choice(["attention", "latent_attention", "mlstm"])
+        mlp = None if rng.random() < 0.2 else {"kind": "dense", "ff": rng.choice([128, 200, 384])}
+        if kind == "attention" and sources and rng.random() < 0.5:
+            source = rng.choice(sources)
+            mixer = dict(layers[source]["mixer"], scale=rng.uniform(0.05, 0.3), kv_from=source)
+        elif kind == "attention":
+            groups = rng.choice([1, 2, 3, 4])
+            d = rng.choice([16, 32, 40, 64, 96])
+            mixer = {"heads": groups * rng.choice([1, 2, 3]), "kv_heads": groups, "dim": d, "vdim": d if rng.random() < 0.5 else rng.choice([16, 24, 64]),
+                     "scale": rng.uniform(0.05, 0.3)}
+            if rng.random() < 0.7:
+                mixer["q_temp"] = {"coef": rng.uniform(0.1, 1.0), "every": rng.choice([1, 7, 32, 64])}
+            sources.append(i)
+        elif kind == "latent_attention":
+            dr = rng.choice([8, 16, 32])
+            mixer = {"heads": rng.choice([2, 4, 6, 12, 20]), "dim": rng.choice([16, 32, 64]), "rot_dim": dr, "vdim": rng.choice([16, 32, 80]),
+                     "q_rank": rng.choice([32, 64, 96]), "kv_rank": rng.choice([32, 48, 100, 128]), "scale": rng.uniform(0.05, 0.2),
+                     "rot": {"base": rng.choice([10000.0, 500.0]), "dims": dr,
+                             "scaling": {"factor": rng.choice([2.0, 8.0]), "original": rng.choice([64, 512]), "fast": 32.0, "slow": 1.0}},
+                     "mask": {"size": rng.choice([1, 5, 16, 17, 64, 100, 300])}}
+        else:
+            mixer = {"heads": rng.choice([1, 2, 4]), "dim": rng.choice([16, 48, 64, 160]), "vdim": rng.choice([16, 48, 100]), "gate_cap": rng.choice([5.0, 15.0])}
+        layers.append({"type": kind, "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Rerizen", "vocab": rng.choice([300, 512]), "width": rng.choice([96, 128, 192]), "streams": rng.choice([1, 2, 3, 4]),
+            "logit_scale": rng.choice([0.25, 1.0, 3.0]), "norm": {"eps": rng.choice([1e-5, 1e-6])}, "layers": layers}
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_models_drawn_at_random(tmp_path, seed):
+    """Sizes, order of layers and constants drawn at random; whole prompts, portions and mixed batches in float32."""
+    import random
+
+    from kipp_amd.weights import write_random_model
+    cfg = random_configuration(random.Random(seed))
+    folder = write_random_model(str(tmp_path / "drawn"), cfg, seed=seed, dtype="float32")
+    requests = {f"r{i}": H.random_tokens(seed * 10 + i, n, cfg["vocab"]) for i, n in enumerate([1, 23, 97, 180])}
+    for maker in (H.whole, H.changing_portions, lambda r: H.mixed(r, seed=seed)):
+        got = H.replay(engine_of(folder, "float32", max_requests=4), requests, maker(requests))
+        for rid, toks in requests.items():
+            close(got[rid], plain_logits(folder, toks), 2e-8, f"drawn {seed}/{rid}: {json.dumps(cfg)}")
+
+
 def test_recorded_steps_of_a_changing_batch(folders):
     """Three requests decode together from recorded steps while the window passes page borders and the memories go on in
     their slots; one ends early and the batch goes on at another size."""
