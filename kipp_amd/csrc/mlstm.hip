@@ -22,7 +22,7 @@
 //         walked out of LDS, the next one's k, q, v and gate pre-activations are on their way from memory into
 //         registers; when a chunk is put into LDS the first wave takes the gates of its tokens (tanh and logarithms a lane a
 //         token, the running maximum in token order, the exponentials a lane a token again), so the walk itself is
-//         multiply-adds.
+//         multiply-adds, and the sums over a column's lanes are data-parallel moves inside the wave, not trips through LDS.
 //         The order of a token's operations does not depend on where its chunk begins: a position's bits are the
 //         same however the prompt was cut.
 // finish  every head of a token divided by its root mean square, times the norm's weight, times sigmoid(gate),
@@ -36,6 +36,28 @@
 #define SCAN_THREADS 256
 #define SCAN_GROUP 8
 #define SCAN_STAGE 4096     // most numbers of k (and of q) that a chunk of tokens stages: 16 a thread
+
+// v + the v of the lane whose number differs in one bit, for bits 0 to 3 by the data-parallel moves inside a row of 16
+// lanes (no trip through LDS): neighbours in a quad, the other pair of a quad, the other quad of a half row (a mirror
+// inside 8 lanes, where every lane of a quad already holds the quad's sum), the other half row (a mirror inside 16).
+template <int STEP>
+__device__ __forceinline__ float lane_pair_sum(float v) {
+    constexpr int ctrl = STEP == 1 ? 0xB1 : (STEP == 2 ? 0x4E : (STEP == 4 ? 0x141 : 0x140));
+    if constexpr (STEP <= 8) return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, 0xF, 0xF, true));
+    else return v + __shfl_xor(v, STEP, KIPP_WAVE);
+}
+
+// The sum over the PARTS lanes of a column, in every one of them: pairs, pairs of pairs, ...
+template <int PARTS>
+__device__ __forceinline__ float column_sum(float v) {
+    if constexpr (PARTS >= 2) v = lane_pair_sum<1>(v);
+    if constexpr (PARTS >= 4) v = lane_pair_sum<2>(v);
+    if constexpr (PARTS >= 8) v = lane_pair_sum<4>(v);
+    if constexpr (PARTS >= 16) v = lane_pair_sum<8>(v);
+    if constexpr (PARTS >= 32) v = lane_pair_sum<16>(v);
+    if constexpr (PARTS >= 64) v = lane_pair_sum<32>(v);
+    return v;
+}
 
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.0f) - log1pf(expf(-fabsf(z))); }
 
@@ -166,9 +188,9 @@ __global__ void __launch_bounds__(SCAN_THREADS) mlstm_scan_kernel(
         __syncthreads();
         const int n_next = min(chunk, count - c0 - chunk);
         if (n_next > 0) fetch(c0 + chunk, n_next);
-        // eight tokens at a time: the gates' chain first (one maximum and three exponentials a token, no lane waits for
-        // another), then the multiply-adds over a lane's rows, then the exchanges between the lanes of a column for all
-        // eight together (each exchange waits as long as a read of LDS; eight of them wait together)
+        // eight tokens at a time: their gates out of LDS, then the multiply-adds over a lane's rows, then the sums over the
+        // lanes of a column for all eight (data-parallel moves inside a row of 16 lanes; only a column of 64 lanes takes
+        // its last two steps through LDS)
         for (int t8 = 0; t8 < n_tok; t8 += SCAN_GROUP) {
             float keep[SCAN_GROUP], take[SCAN_GROUP], floor_p[SCAN_GROUP], num_p[SCAN_GROUP], den_p[SCAN_GROUP];
 #pragma unroll
@@ -193,7 +215,7 @@ __global__ void __launch_bounds__(SCAN_THREADS) mlstm_scan_kernel(
                         *reinterpret_cast<float4*>(qq + r) = *reinterpret_cast<const float4*>(q_t + r);
                     }
                     constexpr int RUNS = ROWS / BASE;
-                    static_assert(RUNS == 1 || RUNS == 2 || RUNS == 4, "runs of rows");
+                    static_assert(RUNS == 1 || RUNS == 2 || RUNS == 4 || RUNS == 8, "runs of rows");
                     float num[RUNS], den[RUNS];
 #pragma unroll
                     for (int g = 0; g < RUNS; ++g) num[g] = den[g] = 0.0f;
@@ -204,17 +226,21 @@ __global__ void __launch_bounds__(SCAN_THREADS) mlstm_scan_kernel(
                         num[r / BASE] = fmaf(S[r], qq[r], num[r / BASE]);
                         den[r / BASE] = fmaf(nv[r], qq[r], den[r / BASE]);
                     }
-                    num_p[u] = RUNS == 4 ? (num[0] + num[1]) + (num[RUNS / 2] + num[RUNS - 1]) : (RUNS == 2 ? num[0] + num[RUNS - 1] : num[0]);
-                    den_p[u] = RUNS == 4 ? (den[0] + den[1]) + (den[RUNS / 2] + den[RUNS - 1]) : (RUNS == 2 ? den[0] + den[RUNS - 1] : den[0]);
+#pragma unroll
+                    for (int w = 1; w < RUNS; w <<= 1)
+#pragma unroll
+                        for (int i = 0; i + w < RUNS; i += 2 * w) {
+                            num[i] += num[i + w];
+                            den[i] += den[i + w];
+                        }
+                    num_p[u] = num[0];
+                    den_p[u] = den[0];
                 }
             }
 #pragma unroll
-            for (int off = 1; off < PARTS; off <<= 1) {
-#pragma unroll
-                for (int u = 0; u < SCAN_GROUP; ++u) {
-                    num_p[u] += __shfl_xor(num_p[u], off, KIPP_WAVE);
-                    den_p[u] += __shfl_xor(den_p[u], off, KIPP_WAVE);
-                }
+            for (int u = 0; u < SCAN_GROUP; ++u) {
+                num_p[u] = column_sum<PARTS>(num_p[u]);
+                den_p[u] = column_sum<PARTS>(den_p[u]);
             }
             if (live && part == 0) {
 #pragma unroll
